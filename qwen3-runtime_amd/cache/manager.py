@@ -44,6 +44,7 @@ class _Group:
     pool: PagePool
     page_size: int
     window: int | None
+    chunk: int | None = None
     tables: dict[Hashable, list[int]] = field(default_factory=dict)
     # index of the first table entry that still holds a page
     first_live: dict[Hashable, int] = field(default_factory=dict)
@@ -85,7 +86,7 @@ class CacheManager:
             if spec.paged:
                 key = spec.group_key()
                 if key not in by_key:
-                    by_key[key] = _Group(key, spec, [], PagePool(num_pages), self.page_size, spec.window)
+                    by_key[key] = _Group(key, spec, [], PagePool(num_pages), self.page_size, spec.window, spec.chunk)
                     self.groups.append(by_key[key])
                 by_key[key].cache_ids.append(cid)
                 self._group_of_cache[cid] = self.groups.index(by_key[key])
@@ -120,11 +121,20 @@ class CacheManager:
         total = 0
         for spec in self.specs:
             if spec.paged:
-                seen = sum(n if spec.window is None else min(n, spec.window) for n in kv_lens)
+                seen = sum(self._visible(spec, n) for n in kv_lens)
                 total += seen * spec.elements_per_token() * width
         for state in self._state_of_cache.values():
             total += len(kv_lens) * state[0].numel() * state.element_size()
         return total
+
+    @staticmethod
+    def _visible(spec: CacheSpec, length: int) -> int:
+        """Keys that the newest of ``length`` tokens sees in a cache of ``spec``."""
+        if spec.window is not None:
+            return min(length, spec.window)
+        if spec.chunk is not None and length > 0:
+            return (length - 1) % spec.chunk + 1
+        return length
 
     @property
     def num_pages(self) -> int:
@@ -147,8 +157,12 @@ class CacheManager:
             if g.window is not None:
                 # `window` consecutive positions touch at most this many pages
                 need = min(need, (g.window - 1 + g.page_size - 1) // g.page_size + 1)
+            if g.chunk is not None:
+                # a chunk's positions likewise (it need not begin where a page begins)
+                need = min(need, (g.chunk - 1 + g.page_size - 1) // g.page_size + 1)
             if need > g.pool.num_pages:
-                what = "" if g.window is None else f" (window {g.window})"
+                what = f" (window {g.window})" if g.window is not None else \
+                    f" (chunks of {g.chunk})" if g.chunk is not None else ""
                 return False, (f"request length {length} needs {need} cache pages in group {i}{what}; "
                                f"the pool has {g.pool.num_pages}")
         return True, ""
@@ -222,16 +236,20 @@ class CacheManager:
         return returned
 
     def commit(self, rid: Hashable, num_tokens: int) -> None:
-        """``num_tokens`` more tokens are stored. Window groups give back what no query sees."""
+        """``num_tokens`` more tokens are stored. Window and chunk groups give back what no query sees."""
         new_len = self._length[rid] + num_tokens
         if new_len > self._reserved[rid]:
             raise AssertionError(f"request {rid!r} stored {new_len} tokens but reserved {self._reserved[rid]}")
         self._length[rid] = new_len
         for g in self.groups:
-            if g.window is None:
+            if g.window is not None:
+                # the next query sits at position >= new_len and sees keys > its position - window
+                first_needed = new_len - g.window + 1
+            elif g.chunk is not None:
+                # ... or the keys of its own chunk, which begins no earlier than new_len's
+                first_needed = new_len - new_len % g.chunk
+            else:
                 continue
-            # the next query sits at position >= new_len and sees keys > its position - window
-            first_needed = new_len - g.window + 1
             table = g.tables[rid]
             i = g.first_live[rid]
             while i < len(table) and (i + 1) * g.page_size <= first_needed:

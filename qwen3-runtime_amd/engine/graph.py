@@ -106,8 +106,8 @@ class DecodeGraph:
     def _advance(self, rids, starts) -> None:
         """The same requests one token further (the usual decode step): the host buffer is brought
         up to date in place, but for the ids. Positions and lengths one up, the slots of the new
-        positions, and a block-table entry where a request has begun a page; groups with a window
-        (whose pages are given back as the window passes) get their tables written afresh. The
+        positions, and a block-table entry where a request has begun a page; groups with a window or a chunk
+        (whose pages are given back as the window passes, or when a chunk ends) get their tables written afresh. The
         pages of the new positions must be reserved."""
         cache = self.runner.cache
         self.copied.synchronize()  # the previous copy has left the host buffer
@@ -118,7 +118,7 @@ class DecodeGraph:
         for gi, g in enumerate(cache.groups):
             table = view[f"table{gi}"]
             page_index = pos // g.page_size
-            if g.window is not None:
+            if g.window is not None or g.chunk is not None:
                 cache.fill_tables(gi, rids, table)
             else:
                 for i in np.nonzero(pos % g.page_size == 0)[0]:

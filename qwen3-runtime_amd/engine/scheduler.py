@@ -52,7 +52,7 @@ class Scheduler:
         if longest - 1 > self.max_model_len:
             raise RuntimeError(
                 f"request length {longest} exceeds the model's limit of {self.max_model_len} positions")
-        # per group of caches: one that keeps a window of keys needs the window's pages only
+        # per group of caches: one that keeps a window or a chunk of keys needs that one's pages only
         fits, why_not = self.cache.can_ever_hold(longest)
         if not fits:
             raise RuntimeError(why_not)

@@ -1,6 +1,6 @@
 """Layer parts. Importing this package registers the shipped kinds."""
 
-from . import attention, block, embedding, mlp, norm, rope  # noqa: F401
+from . import attention, block, embedding, mlp, moe, norm, rope  # noqa: F401
 from .base import (  # noqa: F401
     Block,
     CacheView,
@@ -12,6 +12,7 @@ from .base import (  # noqa: F401
     PositionEncoding,
     StepContext,
     StepCost,
+    StreamUpdate,
 )
 from .model import DecoderModel, build_part  # noqa: F401
 from .plan import CacheSpec, LayerSpec, ModelPlan, PagedStream, PartSpec, RunStep, TensorDecl  # noqa: F401

@@ -10,11 +10,21 @@ cache, output projection. Query head ``h`` reads key/value head ``h // g``,
 to the query at position ``i`` iff ``j <= i`` (and ``j > i - window`` when the
 mixer has a window); softmax in float32
 (reference: qwen3_runtime/attention/pytorch.py:12-47).
+
+Options beyond that form, each a constructor argument: values of another size than keys
+(``value_dim``); the q/k norm without weights (``qk_norm_weight=False``: the heads are divided
+by their root mean square); a fixed score ``scale``; a cap on the scaled scores,
+``softcap * tanh(score / softcap)``, before the softmax; a mask of chunks instead of a window
+(``chunk``: key ``j`` is visible iff ``j <= i`` and ``j // chunk == i // chunk``, chunks counted
+from position 0 of the sequence); an output gate (``output_gate``: one more projection ``g`` of
+the mixer's input, whose sigmoid multiplies the concatenated heads before the output projection).
 """
 
 from __future__ import annotations
 
 import math
+
+import torch
 
 from ..registry import part_class, register_part
 from .base import Mixer
@@ -33,6 +43,11 @@ class GroupedQueryAttention(Mixer):
         position: PartSpec | None = None,
         window: int | None = None,
         scale: float | None = None,
+        value_dim: int | None = None,
+        qk_norm_weight: bool = True,
+        softcap: float | None = None,
+        chunk: int | None = None,
+        output_gate: bool = False,
         tensors=None,
     ):
         super().__init__(tensors)
@@ -44,6 +59,13 @@ class GroupedQueryAttention(Mixer):
         self.head_dim = int(head_dim)
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.window = None if window is None else int(window)
+        self.chunk = None if chunk is None else int(chunk)
+        if self.window is not None and self.chunk is not None:
+            raise ValueError("a mixer has a window or a mask of chunks, not both")
+        self.value_dim = self.head_dim if value_dim is None else int(value_dim)
+        self.qk_norm_weight = bool(qk_norm_weight)
+        self.softcap = None if softcap is None else float(softcap)
+        self.output_gate = bool(output_gate)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = None
         if position is not None:
@@ -54,17 +76,20 @@ class GroupedQueryAttention(Mixer):
         return (self.position,) if self.position is not None else ()
 
     def cache_spec(self):
-        return CacheSpec("paged_kv", heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window)
+        return CacheSpec("paged_kv", heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window,
+                         chunk=self.chunk, value_dim=None if self.value_dim == self.head_dim else self.value_dim)
 
     def tensor_decls(self):
-        h, d = self.hidden_size, self.head_dim
+        h, d, dv = self.hidden_size, self.head_dim, self.value_dim
         decls = [
             TensorDecl(self._name("q"), (self.num_heads * d, h)),
             TensorDecl(self._name("k"), (self.num_kv_heads * d, h)),
-            TensorDecl(self._name("v"), (self.num_kv_heads * d, h)),
-            TensorDecl(self._name("o"), (h, self.num_heads * d)),
+            TensorDecl(self._name("v"), (self.num_kv_heads * dv, h)),
+            TensorDecl(self._name("o"), (h, self.num_heads * dv)),
         ]
-        if self.qk_norm_eps is not None:
+        if self.output_gate:
+            decls.append(TensorDecl(self._name("g"), (self.num_heads * dv, h)))
+        if self.qk_norm_eps is not None and self.qk_norm_weight:
             decls += [
                 TensorDecl(self._name("q_norm"), (d,), init="norm"),
                 TensorDecl(self._name("k_norm"), (d,), init="norm"),
@@ -72,41 +97,67 @@ class GroupedQueryAttention(Mixer):
         return decls
 
     def load(self, fetch):
-        self.qkv = fetch.fused([self._name("q"), self._name("k"), self._name("v")], dim=0)
+        # one product for q | k | v (| gate): the gate reads the same input
+        names = [self._name("q"), self._name("k"), self._name("v")] + ([self._name("g")] if self.output_gate else [])
+        self.qkv = fetch.fused(names, dim=0)
         self.o = fetch.matrix(self._name("o"))
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_weight:
             self.q_norm = fetch.vector_f32(self._name("q_norm"))
             self.k_norm = fetch.vector_f32(self._name("k_norm"))
+        elif self.qk_norm_eps is not None:  # a norm without weights: weights of one
+            self.q_norm = self.k_norm = fetch.constant(torch.ones(self.head_dim, dtype=torch.float32))
 
     def step_cost(self, spans, rows, elem_bytes):
         cost = super().step_cost(spans, rows, elem_bytes)  # the four projections
         for q, kv in spans:  # scores and weighted values: 4 D operations per (query head, visible key)
             first = kv - q
-            pairs = sum(min(first + i + 1, self.window or kv) for i in range(q)) if self.window else \
-                q * first + q * (q + 1) // 2
-            cost.flop += 4.0 * self.num_heads * self.head_dim * pairs
+            if self.window:
+                pairs = sum(min(first + i + 1, self.window) for i in range(q))
+            elif self.chunk:
+                pairs = sum((first + i) % self.chunk + 1 for i in range(q))
+            else:
+                pairs = q * first + q * (q + 1) // 2
+            cost.flop += 2.0 * self.num_heads * (self.head_dim + self.value_dim) * pairs
         return cost
 
     def forward(self, ctx, x, cache):
         ops = ctx.ops
-        nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        nq, nkv, d, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
         qkv = ops.linear(x, self.qkv)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
         fused = self.position is None or self.position.fused_form == "neox_full"
         inv_freq = None if self.position is None or not fused else self.position.inv_freq
-        if fused and ops.fuses_decode_attention(ctx, qkv, nq, nkv, d, cache):
+        # what only some designs have travels by name, and only where it is set
+        more = {}
+        if dv != d:
+            more["value_dim"] = dv
+        if self.chunk is not None:
+            more["chunk"] = self.chunk
+        if self.softcap is not None:
+            more["softcap"] = self.softcap
+        gate_width = nq * dv if self.output_gate else 0
+        if gate_width:
+            # the gate's columns stay where the product put them: the attention reads them there
+            more["gate"] = qkv[:, qkv.shape[1] - gate_width:]
+        if fused and ops.fuses_decode_attention(ctx, qkv, nq, nkv, d, cache, **more):
             # a step of single tokens: all of it inside the attention kernel
             attn = ops.decode_attention(qkv, cache, ctx, nq, nkv, d, self.scale, self.window,
                                         self.q_norm, self.k_norm, eps, inv_freq,
-                                        None if self.position is None else self.position.angles_key)
+                                        None if self.position is None else self.position.angles_key, **more)
             return ops.linear_for_residual(attn, self.o)
         if fused:
             # norm, rotation and the cache write in one pass over qkv
+            shape = {k: more[k] for k in ("value_dim",) if k in more}
+            if gate_width:
+                shape["extra"] = gate_width
             q = ops.qk_norm_rope_store(
                 qkv, nq, nkv, d, self.q_norm, self.k_norm, eps, inv_freq, ctx.positions,
                 cache if cache.writes else None, ctx=ctx,
-                angles_key=None if self.position is None else self.position.angles_key,
+                angles_key=None if self.position is None else self.position.angles_key, **shape,
             )
+        elif dv != d or gate_width:
+            raise NotImplementedError("a position encoding without a fused form, with values of another size "
+                                      "than keys or an output gate: the unfused steps do not take these")
         else:
             # an encoding the fused kernel has no form for: norm, let it rotate, then store
             q, k, v = ops.qk_norm_split(qkv, nq, nkv, d, self.q_norm, self.k_norm, eps)
@@ -114,5 +165,5 @@ class GroupedQueryAttention(Mixer):
             if cache.writes:
                 ops.kv_store(k, v, cache)
             q = q.reshape(ctx.num_tokens, nq * d)
-        attn = ops.paged_attention(q, cache, ctx, nq, nkv, d, self.scale, self.window)
+        attn = ops.paged_attention(q, cache, ctx, nq, nkv, d, self.scale, self.window, **more)
         return ops.linear_for_residual(attn, self.o)

@@ -8,8 +8,10 @@ configuration the numbers came from.
 Roles and the call each must answer (``T`` tokens of this step, ``H`` width):
 
 * embedding      ``forward(ctx, ids[T] int32) -> residual[T, H] float32``
-* norm           ``forward(ctx, residual[T, H] float32, delta[T, H] | None, rows=None) -> [T|R, H]``
-                 adds ``delta`` into ``residual`` in place, then normalises
+* norm           ``forward(ctx, residual[T, H] float32, delta[T, H] | None, rows=None, read=None) -> [T|R, H]``
+                 adds ``delta`` into ``residual`` in place, then normalises; over several
+                 residual streams ``[T, S, H]`` ``delta`` is a ``StreamUpdate`` and ``read``
+                 the weights ``[S]`` of the sum of streams that is normalised
 * mixer          ``forward(ctx, x[T, H], cache: CacheView | None) -> [T, H]``
 * feed_forward   ``forward(ctx, x[T, H]) -> [T, H]``
 * position       ``rotate(ctx, q[T, nq, D], k[T, nkv, D]) -> (q, k)``
@@ -149,6 +151,17 @@ class Block(Part):
 
 
 @dataclass
+class StreamUpdate:
+    """What a sub-layer leaves to be done to ``S`` residual streams ``x[T, S, H]``:
+    ``new[:, t] = sum_s mix[s, t] * x[:, s] + out[t] * y``, every new stream from the old ones.
+    Like a plain ``delta`` it is applied by the norm that comes next."""
+
+    y: torch.Tensor    # [T, H], or float32 planes [P, T, H] whose sum it is
+    mix: torch.Tensor  # float32 [S, S], indexed [from, to]
+    out: torch.Tensor  # float32 [S]
+
+
+@dataclass
 class GroupView:
     """One cache group's view of this step's batch (device tensors).
 
@@ -162,6 +175,8 @@ class GroupView:
     window: int | None
     block_table: torch.Tensor
     slots: torch.Tensor
+    # keys are kept for the chunk of this many positions that the newest token lies in
+    chunk: int | None = None
 
 
 @dataclass

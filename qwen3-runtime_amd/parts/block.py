@@ -1,4 +1,5 @@
-"""Arrangement of a layer's parts: the pre-norm residual block.
+"""Arrangements of a layer's parts: the pre-norm residual block, over one residual stream or
+over several (hyper-connections).
 
 ``x += mixer(norm_in(x)); x += feed_forward(norm_post(x))``: the form the
 reference's oracle writes (tests/cpu/reference_qwen3.py:79-110) and its model
@@ -11,7 +12,8 @@ with the norm that follows it without a block knowing its neighbour.
 from __future__ import annotations
 
 from ..registry import register_part
-from .base import Block
+from .base import Block, StreamUpdate
+from .plan import TensorDecl
 
 
 @register_part("block", "pre_norm")
@@ -23,13 +25,78 @@ class PreNormBlock(Block):
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norm_in = norms["input"]
-        self.norm_post = norms["post_mixer"]
+        self.norm_post = norms.get("post_mixer")
 
     def children(self):
-        return (self.norm_in, self.mixer, self.norm_post, self.feed_forward)
+        return tuple(p for p in (self.norm_in, self.mixer, self.norm_post, self.feed_forward) if p is not None)
 
     def forward(self, ctx, residual, delta, cache):
         x = self.norm_in.forward(ctx, residual, delta)
         mixed = self.mixer.forward(ctx, x, cache)
+        if self.feed_forward is None:  # a layer of a mixer alone
+            return residual, mixed
         x = self.norm_post.forward(ctx, residual, mixed)
         return residual, self.feed_forward.forward(ctx, x)
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionBlock(Block):
+    """Pre-norm sub-layers over ``streams`` residual streams ``x[T, S, H]`` that all start as the
+    embedding. Sub-layer ``q`` (1 the mixer, 2 the feed-forward) reads ``u = sum_s in_q[s] x_s``,
+    computes ``y = f(norm(u))``, and leaves ``x_t <- sum_s mix_q[s, t] x_s + out_q[t] y`` to the
+    norm that comes next, which applies it in the pass in which it reads the streams: the one
+    kernel between two sub-layers does the write of one and the read of the other. A block without
+    feed-forward has the first sub-layer only. The model's last norm sums the streams."""
+
+    norm_names = ("input", "post_mixer")
+
+    def __init__(self, mixer, feed_forward, norms, streams: int, tensors=None):
+        super().__init__(tensors)
+        self.streams = int(streams)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norm_in = norms["input"]
+        self.norm_post = norms.get("post_mixer")
+        if (feed_forward is None) != (self.norm_post is None):
+            raise ValueError("a feed-forward and the norm in front of it come together")
+        self.coeff: dict[str, object] = {}
+
+    def children(self):
+        return tuple(p for p in (self.norm_in, self.mixer, self.norm_post, self.feed_forward) if p is not None)
+
+    def _sublayers(self):
+        return ("1",) if self.feed_forward is None else ("1", "2")
+
+    def tensor_decls(self):
+        s = self.streams
+        decls = []
+        for q in self._sublayers():
+            decls += [TensorDecl(self._name(f"in{q}"), (s,), init="norm"),
+                      TensorDecl(self._name(f"out{q}"), (s,), init="norm"),
+                      TensorDecl(self._name(f"mix{q}"), (s, s), init="mixing")]
+        return decls
+
+    def load(self, fetch):
+        for q in self._sublayers():
+            for name in (f"in{q}", f"out{q}", f"mix{q}"):
+                self.coeff[name] = fetch.vector_f32(self._name(name))
+
+    def step_cost(self, spans, rows, elem_bytes):
+        cost = super().step_cost(spans, rows, elem_bytes)
+        cost.flop = 0.0  # coefficients, not matrices that multiply tokens
+        return cost
+
+    def forward(self, ctx, residual, delta, cache):
+        if residual.dim() == 2:
+            # the one stream that the embedding began: every stream starts as a copy of it
+            if delta is not None:
+                raise ValueError("the residual streams begin at the embedding, with nothing pending")
+            t, h = residual.shape
+            residual = residual[:, None, :].expand(t, self.streams, h).contiguous()
+        c = self.coeff
+        x = self.norm_in.forward(ctx, residual, delta, read=c["in1"])
+        pending = StreamUpdate(self.mixer.forward(ctx, x, cache), c["mix1"], c["out1"])
+        if self.feed_forward is None:
+            return residual, pending
+        x = self.norm_post.forward(ctx, residual, pending, read=c["in2"])
+        return residual, StreamUpdate(self.feed_forward.forward(ctx, x), c["mix2"], c["out2"])

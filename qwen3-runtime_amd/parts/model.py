@@ -33,7 +33,7 @@ class DecoderModel:
         self.blocks = []
         for layer in plan.layers:
             mixer = build_part("mixer", layer.mixer)
-            ff = build_part("feed_forward", layer.feed_forward)
+            ff = None if layer.feed_forward is None else build_part("feed_forward", layer.feed_forward)
             norms = {name: build_part("norm", spec) for name, spec in layer.norms.items()}
             block_cls = part_class("block", layer.block.kind)
             self.blocks.append(

@@ -33,7 +33,8 @@ class TensorDecl:
     """One tensor a part reads from the model file.
 
     ``init`` tells the random-weights mode how to draw it: ``"matrix"`` and
-    ``"embedding"`` are zero-mean normal, ``"norm"`` is a scale around one.
+    ``"embedding"`` are zero-mean normal, ``"norm"`` is a scale around one, ``"mixing"``
+    a square matrix around the identity.
     ``storage`` is ``"float"`` (stored as bfloat16, float32 or float16) or ``"int"``
     (an integer table, held as int32; drawn as zeros in the random-weights mode unless
     ``init`` is ``"index:<n>"``, uniform in ``[0, n)``).
@@ -70,7 +71,9 @@ class CacheSpec:
     """What one cache owner keeps between steps.
 
     ``kind == "paged_kv"``: keys and values for every token (or the last
-    ``window`` tokens), ``heads`` x ``head_dim`` keys and ``heads`` x ``value_dim``
+    ``window`` tokens, or, with ``chunk``, the tokens of the chunk of ``chunk``
+    positions, counted from position 0, that the newest token lies in),
+    ``heads`` x ``head_dim`` keys and ``heads`` x ``value_dim``
     values (``head_dim`` when None), held in pages; the values transposed within a
     page. ``kind == "paged"``: any other set of per-token tensors, named by
     ``streams`` (one latent vector per token, say), with the same pages, tables and
@@ -86,6 +89,14 @@ class CacheSpec:
     dtype: str = "model"
     value_dim: int | None = None
     streams: tuple[PagedStream, ...] = ()
+    chunk: int | None = None
+
+    def __post_init__(self) -> None:
+        if self.window is not None and self.chunk is not None:
+            raise ValueError("a cache keeps a window of keys or a chunk of them, not both")
+        for name in ("window", "chunk"):
+            if getattr(self, name) is not None and getattr(self, name) < 1:
+                raise ValueError(f"{name} must be positive, got {getattr(self, name)}")
 
     @property
     def paged(self) -> bool:
@@ -109,17 +120,18 @@ class CacheSpec:
     def group_key(self) -> tuple:
         """Caches with equal keys share pages' geometry and lifetime, hence a pool."""
         if self.paged:
-            return ("paged", self.page_streams(), self.window)
+            return ("paged", self.page_streams(), self.window, self.chunk)
         return ("state", tuple(self.shape), self.dtype)
 
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a block arrangement over a mixer, a feed-forward and norms."""
+    """One layer: a block arrangement over a mixer, a feed-forward (None: the layer has
+    none) and norms."""
 
     block: PartSpec
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: PartSpec | None
     norms: Mapping[str, PartSpec]
 
 

@@ -49,7 +49,8 @@ def architecture_names() -> list[str]:
 def architecture_for(raw_config: Mapping[str, Any]) -> Architecture:
     """Pick the architecture a config.json names, or say which ones exist."""
     _load_builtin()
-    names = raw_config.get("architectures") or []
+    # a list under "architectures", or one name under "architecture"
+    names = raw_config.get("architectures") or raw_config.get("architecture") or []
     if isinstance(names, str):
         names = [names]
     for name in names:
@@ -64,7 +65,7 @@ def register_preset(name: str, raw_config: Mapping[str, Any], page_size: int = 1
     """A named configuration (a config.json as a dict, ``architectures`` included) that the
     entry points build with random weights: ``--preset NAME`` on the command line, and the
     model ``LLM(None)`` makes is the first one registered."""
-    if not raw_config.get("architectures"):
+    if not (raw_config.get("architectures") or raw_config.get("architecture")):
         raise ValueError(f"preset {name!r}: the configuration names no architecture")
     _PRESETS[name] = (dict(raw_config), int(page_size))
 
@@ -132,4 +133,5 @@ def _load_builtin() -> None:
         return
     _loaded = True
     from . import parts  # noqa: F401  (registers part kinds)
-    from .models import qwen3  # noqa: F401  (registers Qwen3ForCausalLM)
+    from .models import qwen3  # noqa: F401  (registers Qwen3ForCausalLM; its presets come first)
+    from .models import deginex  # noqa: F401  (registers Deginex)

@@ -75,7 +75,7 @@ class RandomSource:
     values do not depend on which other tensors exist or on the order they are
     asked for. ``"matrix"`` and ``"embedding"`` tensors are N(0, std);
     ``"norm"`` tensors are ``1 + N(0, norm_jitter)`` (all ones when the jitter
-    is zero). Values are rounded to ``store_dtype``. Integer tables
+    is zero), ``"mixing"`` matrices the identity plus ``N(0, norm_jitter)``. Values are rounded to ``store_dtype``. Integer tables
     (``storage="int"``) are int32: zeros, or uniform in ``[0, n)`` for ``init="index:<n>"``.
     """
 
@@ -118,6 +118,8 @@ class RandomSource:
         x = torch.randn(decl.shape, generator=gen, dtype=torch.float32, device=device)
         if decl.init == "norm":
             x = 1.0 + self.norm_jitter * x
+        elif decl.init == "mixing":
+            x = torch.eye(decl.shape[0], decl.shape[1], dtype=torch.float32, device=device) + self.norm_jitter * x
         else:
             x = self.std * x
         return x.to(self.store_dtype)

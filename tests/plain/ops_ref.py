@@ -77,11 +77,13 @@ def kv_store(k, v, k_cache, v_cache, slots, page_size):
 
 
 def qk_norm_rope_store(qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions,
-                       k_cache=None, v_cache=None, slots=None, page_size=None, compute=torch.float32):
+                       k_cache=None, v_cache=None, slots=None, page_size=None, compute=torch.float32,
+                       value_dim=None):
     t = qkv.shape[0]
+    dv = d if value_dim is None else value_dim
     q = qkv[:, : nq * d].reshape(t, nq, d)
     k = qkv[:, nq * d: (nq + nkv) * d].reshape(t, nkv, d)
-    v = qkv[:, (nq + nkv) * d:].reshape(t, nkv, d)
+    v = qkv[:, (nq + nkv) * d: (nq + nkv) * d + nkv * dv].reshape(t, nkv, dv)
     q = head_rmsnorm(q, q_w, eps, compute)
     k = head_rmsnorm(k, k_w, eps, compute)
     if inv_freq is not None:
@@ -105,10 +107,14 @@ def gather_kv(k_cache, v_cache, table_row, lo, hi, page_size):
 
 
 def paged_attention(q, k_cache, v_cache, cu_q, kv_lens, block_table, page_size, nq, nkv, d,
-                    scale, window=None, compute=torch.float32, round_probs=False):
-    """q [T, nq*D] -> [T, nq*D]. Query row i of a sequence sits at position
-    kv_len - q_len + i and sees keys j <= its position (and > position - window)."""
-    out = torch.zeros_like(q)
+                    scale, window=None, compute=torch.float32, round_probs=False, chunk=None, softcap=None,
+                    value_dim=None, gate=None):
+    """q [T, nq*D] -> [T, nq*Dv]. Query row i of a sequence sits at position
+    kv_len - q_len + i and sees keys j <= its position (and > position - window, or, with
+    ``chunk``, in its own chunk of positions). ``softcap``: scores become cap * tanh(score / cap).
+    ``gate`` [T, nq*Dv]: the output is multiplied by its sigmoid."""
+    dv = d if value_dim is None else value_dim
+    out = torch.zeros((q.shape[0], nq * dv), dtype=q.dtype, device=q.device)
     g = nq // nkv
     cu = [int(x) for x in cu_q]
     for s in range(len(cu) - 1):
@@ -118,6 +124,8 @@ def paged_attention(q, k_cache, v_cache, cu_q, kv_lens, block_table, page_size, 
             continue
         first_pos = kv_len - q_len
         lo = 0 if window is None else max(0, first_pos - window + 1)
+        if chunk is not None:
+            lo = first_pos - first_pos % chunk
         k, v = gather_kv(k_cache, v_cache, block_table[s], lo, kv_len, page_size)
         k = k.to(compute).repeat_interleave(g, dim=1)
         v = v.to(compute).repeat_interleave(g, dim=1)
@@ -128,12 +136,77 @@ def paged_attention(q, k_cache, v_cache, cu_q, kv_lens, block_table, page_size, 
         ok = kpos <= qpos
         if window is not None:
             ok = ok & (kpos > qpos - window)
+        if chunk is not None:
+            ok = ok & (kpos // chunk == qpos // chunk)
+        if softcap is not None:
+            scores = softcap * torch.tanh(scores / softcap)
         scores = scores.masked_fill(~ok, float("-inf"))
         probs = torch.softmax(scores, dim=-1)
         if round_probs:
             probs = probs.to(q.dtype).to(compute)
-        ctx = torch.einsum("hqk,khd->qhd", probs, v)
-        out[a:b] = ctx.reshape(q_len, nq * d).to(q.dtype)
+        ctx = torch.einsum("hqk,khd->qhd", probs, v).reshape(q_len, nq * dv)
+        if gate is not None:
+            ctx = ctx * torch.sigmoid(gate[a:b].to(compute))
+        out[a:b] = ctx.to(q.dtype)
+    return out
+
+
+def mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows=None, compute=torch.float32):
+    """Residual streams [T, S, H] (or one stream [T, H]) float32. ``update``: None, a plain delta
+    (one stream only), or an object with ``y`` [T, H] (or planes [P, T, H]), ``mix`` [S, S]
+    (indexed [from, to]) and ``out`` [S]: new[:, t] = sum_s mix[s, t] old[:, s] + out[t] y,
+    written back unless ``rows`` is given. Returns the norm (layer norm with ``bias``, RMS norm
+    without) of sum_t read[t] new[:, t] at the rows asked for."""
+    one = streams.dim() == 2
+    x = streams[:, None, :] if one else streams
+    new = x
+    if update is not None:
+        if hasattr(update, "y"):
+            y, mix, out = update.y, update.mix, update.out
+        else:
+            y, mix, out = update, None, None
+        if y.dim() == 3:
+            y = y.to(torch.float32).sum(0)
+        y = y.to(torch.float32)
+        new = x if mix is None else torch.einsum("sr,tsh->trh", mix.to(torch.float32), x)
+        new = new + (y[:, None, :] if out is None else out.to(torch.float32)[None, :, None] * y[:, None, :])
+        if rows is None:
+            x.copy_(new)
+    u = new[:, 0] if read is None else torch.einsum("s,tsh->th", read.to(torch.float32), new)
+    if rows is not None:
+        u = u[rows.long()]
+    u = u.to(compute)
+    if bias is None:
+        y = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * weight.to(compute)
+    else:
+        mu = u.mean(-1, keepdim=True)
+        var = (u - mu).pow(2).mean(-1, keepdim=True)
+        y = (u - mu) * torch.rsqrt(var + eps) * weight.to(compute) + bias.to(compute)
+    return y.to(out_dtype)
+
+
+def route_top(x, router, router_bias, top):
+    """float32 logits x W^T + b; the ``top`` largest per token (ties: the lower index first) and
+    the softmax over those alone. Returns (int32 [T, top], float32 [T, top])."""
+    logits = x.to(torch.float32) @ router.to(torch.float32).T
+    if router_bias is not None:
+        logits = logits + router_bias.to(torch.float32)
+    best, index = torch.topk(logits, top, dim=-1)
+    return index.to(torch.int32), torch.softmax(best, dim=-1)
+
+
+def moe_swiglu(x, gate_up, down, index, weight, compute=torch.float32):
+    """x [T, H]; gate_up [E, 2I, H]; down [E, H, I]; index/weight [T, top] -> [T, H] (float32)."""
+    t, h = x.shape
+    inter = gate_up.shape[1] // 2
+    out = torch.zeros((t, h), dtype=torch.float32, device=x.device)
+    xc = x.to(compute)
+    for j in range(index.shape[1]):
+        for e in index[:, j].unique().tolist():
+            sel = (index[:, j] == e).nonzero()[:, 0]
+            gu = (xc[sel] @ gate_up[e].to(compute).T).to(x.dtype).to(compute)
+            act = (gu[:, :inter] * torch.sigmoid(gu[:, :inter]) * gu[:, inter:]).to(x.dtype).to(compute)
+            out[sel] += weight[sel, j, None] * (act @ down[e].to(compute).T).to(torch.float32)
     return out
 
 
@@ -166,14 +239,24 @@ class TorchOps:
         return linear(x, w, False, self.compute)
 
     def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache, ctx=None,
-                           angles_key=None):
+                           angles_key=None, value_dim=None, extra=0):
         if cache is None:
             return qk_norm_rope_store(qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions,
-                                      compute=self.compute)
+                                      compute=self.compute, value_dim=value_dim)
         return qk_norm_rope_store(qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions,
-                                  cache.k, cache.v, cache.group.slots, cache.group.page_size, self.compute)
+                                  cache.k, cache.v, cache.group.slots, cache.group.page_size, self.compute,
+                                  value_dim=value_dim)
 
-    def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache):
+    def mix_norm(self, streams, update, read, weight, bias, eps, out_dtype, rows=None):
+        return mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows, self.compute)
+
+    def route_top(self, x, router, router_bias, top):
+        return route_top(x, router, router_bias, top)
+
+    def moe_swiglu(self, x, gate_up, down, index, weight):
+        return moe_swiglu(x, gate_up, down, index, weight, self.compute)
+
+    def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache, **more):
         return False  # no one-kernel form of a decode step's attention here: the steps above, in order
 
     def qk_norm_split(self, qkv, nq, nkv, d, q_w, k_w, eps):
@@ -186,9 +269,11 @@ class TorchOps:
     def kv_store(self, k, v, cache):
         kv_store(k, v, cache.k, cache.v, cache.group.slots, cache.group.page_size)
 
-    def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window):
+    def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window, chunk=None, softcap=None, value_dim=None,
+                        gate=None):
         return paged_attention(q, cache.k, cache.v, ctx.cu_q, ctx.kv_lens, cache.group.block_table,
-                               cache.group.page_size, nq, nkv, d, scale, window, self.compute)
+                               cache.group.page_size, nq, nkv, d, scale, window, self.compute, chunk=chunk,
+                               softcap=softcap, value_dim=value_dim, gate=gate)
 
     def swiglu(self, gate_up):
         return swiglu(gate_up, self.compute)
