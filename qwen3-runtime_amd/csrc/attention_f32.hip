@@ -5,8 +5,10 @@
 // maximum and sum (online softmax, float32), and accumulates the context with
 // each lane owning head elements lane, lane + 64, ... Query head h reads key
 // head h / g. The query at position p sees keys j <= p, and j > p - window when
-// a window is set. Cache layout: keys [page, head, offset, D], values
-// [page, head, D, offset].
+// a window is set, or j >= p - p % chunk when a chunk size is. Scores are
+// dot * scale, then, with a cap, cap * tanh(score / cap). Values may have another
+// size Dv than keys; with a gate the output is multiplied by sigmoid(gate). Cache
+// layout: keys [page, head, offset, D], values [page, head, Dv, offset].
 #include "common.h"
 #include <math.h>
 
@@ -21,6 +23,11 @@ struct AttnArgs {
   int table_width;
   int num_tokens, nq, nkv, head_dim, page_size, window;  // window 0: none
   float scale;
+  int chunk;       // 0: none
+  float softcap;   // 0: none
+  int value_dim;   // 0: head_dim
+  const void* gate;  // [T, gate_stride] with nq * Dv columns used, or null
+  long gate_stride;
 };
 
 #define MAX_D 512
@@ -30,7 +37,7 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
   __shared__ float qs[MAX_D];
   const int lane = threadIdx.x;
   const int t = blockIdx.x, h = blockIdx.y;
-  const int D = a.head_dim, ps = a.page_size;
+  const int D = a.head_dim, ps = a.page_size, Dv = a.value_dim;
   const int kvh = h / (a.nq / a.nkv);
   const int pos = a.positions[t];
   const int* table = a.block_table + (size_t)a.seq_of_token[t] * a.table_width;
@@ -38,7 +45,7 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
   for (int i = lane; i < D; i += 64) qs[i] = to_f32<T>(q[i]);
   __syncthreads();
 
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : (a.chunk > 0 ? pos - pos % a.chunk : 0);
   float m = -INFINITY, l = 0.f;
   float acc[MAX_D / 64];
 #pragma unroll
@@ -58,6 +65,7 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32<T>(kr[d]), dot);
       s = dot * a.scale;
+      if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -71,20 +79,25 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
       const float pj = __shfl(p, jj, 64);
       const int pg = __shfl(page, jj, 64);
       const int of = __shfl(off, jj, 64);
-      const T* vr = vc + ((size_t)pg * a.nkv + kvh) * D * ps + of;
+      const T* vr = vc + ((size_t)pg * a.nkv + kvh) * Dv * ps + of;
 #pragma unroll
       for (int i = 0; i < MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
-        if (d < D) acc[i] = fmaf(pj, to_f32<T>(vr[(size_t)d * ps]), acc[i]);
+        if (d < Dv) acc[i] = fmaf(pj, to_f32<T>(vr[(size_t)d * ps]), acc[i]);
       }
     }
   }
-  T* o = (T*)a.out + ((size_t)t * a.nq + h) * D;
+  T* o = (T*)a.out + ((size_t)t * a.nq + h) * Dv;
+  const T* gate = a.gate ? (const T*)a.gate + (size_t)t * a.gate_stride + (size_t)h * Dv : nullptr;
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int i = 0; i < MAX_D / 64; ++i) {
     const int d = lane + 64 * i;
-    if (d < D) o[d] = from_f32<T>(acc[i] * inv);
+    if (d < Dv) {
+      float v = acc[i] * inv;
+      if (gate) v *= 1.0f / (1.0f + expf(-to_f32<T>(gate[d])));
+      o[d] = from_f32<T>(v);
+    }
   }
 }
 
@@ -94,6 +107,10 @@ extern "C" int qrt_attention_f32(const AttnArgs* args, int dtype, hipStream_t st
             "attention: %d query heads do not divide into %d key heads", a.nq, a.nkv);
   QRT_CHECK(a.head_dim > 0 && a.head_dim <= MAX_D, "attention: head size %d is above %d", a.head_dim, MAX_D);
   QRT_CHECK(a.page_size > 0 && a.table_width > 0 && a.window >= 0, "attention: bad page size, table width or window");
+  if (a.value_dim == 0) a.value_dim = a.head_dim;
+  QRT_CHECK(a.value_dim > 0 && a.value_dim <= MAX_D, "attention: value size %d is above %d", a.value_dim, MAX_D);
+  QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a chunk size, not both");
+  QRT_CHECK(a.softcap >= 0.f, "attention: negative score cap");
   QRT_CHECK(a.nq <= 65535, "attention: too many heads");
   if (a.num_tokens == 0) return 0;
   dim3 grid(a.num_tokens, a.nq), block(64);

@@ -303,6 +303,7 @@ struct QkArgs {
   // rope_table makes them. The kernel for many tokens looks them up instead of computing them in
   // every layer (inv_freq and positions are still given: the kernel for few tokens computes).
   const float* rope;
+  int value_dim;  // elements of a value head; 0: head_dim
 };
 
 template <typename T>
@@ -317,16 +318,17 @@ __global__ void qk_norm_rope_store_kernel(QkArgs a) {
 
   if (h >= a.nq + a.nkv) {  // value head: copy
     const int hv = h - a.nq - a.nkv;
-    const T* src = (const T*)a.v_in + (size_t)t * a.v_stride + (size_t)hv * D;
+    const int Dv = a.value_dim;
+    const T* src = (const T*)a.v_in + (size_t)t * a.v_stride + (size_t)hv * Dv;
     if (a.v_out) {
-      T* dst = (T*)a.v_out + ((size_t)t * a.nv + hv) * D;
-      for (int i = lane; i < D; i += 64) dst[i] = src[i];
+      T* dst = (T*)a.v_out + ((size_t)t * a.nv + hv) * Dv;
+      for (int i = lane; i < Dv; i += 64) dst[i] = src[i];
     }
     if (a.slots) {
       const int slot = a.slots[t];
       const int page = slot / a.page_size, off = slot - page * a.page_size;
-      T* dst = (T*)a.v_cache + ((size_t)page * a.nv + hv) * D * a.page_size + off;
-      for (int i = lane; i < D; i += 64) dst[(size_t)i * a.page_size] = src[i];
+      T* dst = (T*)a.v_cache + ((size_t)page * a.nv + hv) * Dv * a.page_size + off;
+      for (int i = lane; i < Dv; i += 64) dst[(size_t)i * a.page_size] = src[i];
     }
     return;
   }
@@ -550,6 +552,8 @@ extern "C" int qrt_qk_norm_rope_store(const QkArgs* args, int dtype, long num_ca
   QRT_CHECK(a.nkv == 0 || a.k_in, "qk_norm_rope_store: key heads without input");
   QRT_CHECK(a.nv == 0 || a.v_in, "qk_norm_rope_store: value heads without input");
   QRT_CHECK(!a.inv_freq || a.positions, "qk_norm_rope_store: rotation without positions");
+  if (a.value_dim == 0) a.value_dim = a.head_dim;
+  QRT_CHECK(a.value_dim > 0, "qk_norm_rope_store: bad value size %d", a.value_dim);
   if (a.slots) {
     QRT_CHECK(a.k_cache && a.v_cache && a.page_size > 0 && num_cache_pages > 0,
               "qk_norm_rope_store: cache write without cache");
@@ -563,7 +567,7 @@ extern "C" int qrt_qk_norm_rope_store(const QkArgs* args, int dtype, long num_ca
   const int D = a.head_dim;
   // few tokens (decoding): the time is the launch and one round of memory latency, and the
   // one-head-per-wave kernel has the shorter chain
-  const bool wide = a.num_tokens >= 32 && D >= 16 && (D & (D - 1)) == 0 && a.q_stride % 8 == 0 && a.k_stride % 8 == 0 &&
+  const bool wide = a.num_tokens >= 32 && D >= 16 && a.value_dim == D && (D & (D - 1)) == 0 && a.q_stride % 8 == 0 && a.k_stride % 8 == 0 &&
                     a.v_stride % 8 == 0 && lined_up(a.q_in) && lined_up(a.k_in) && lined_up(a.v_in) &&
                     lined_up(a.q_out) && lined_up(a.k_out) && lined_up(a.v_out) && lined_up(a.k_cache) &&
                     lined_up(a.v_cache);

@@ -44,6 +44,7 @@ class _QkArgs(Structure):
         ("k_cache", c_void_p), ("v_cache", c_void_p),
         ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int), ("nv", c_int),
         ("head_dim", c_int), ("page_size", c_int), ("eps", c_float), ("rope", c_void_p),
+        ("value_dim", c_int),
     ]
 
 
@@ -53,6 +54,16 @@ class _AttnArgs(Structure):
         ("positions", c_void_p), ("seq_of_token", c_void_p), ("block_table", c_void_p),
         ("table_width", c_int), ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int),
         ("head_dim", c_int), ("page_size", c_int), ("window", c_int), ("scale", c_float),
+        ("chunk", c_int), ("softcap", c_float), ("value_dim", c_int), ("gate", c_void_p), ("gate_stride", c_long),
+    ]
+
+
+class _MixNormArgs(Structure):
+    _fields_ = [
+        ("x_in", c_void_p), ("x_out", c_void_p), ("y", c_void_p), ("mix", c_void_p), ("out_w", c_void_p),
+        ("read", c_void_p), ("weight", c_void_p), ("bias", c_void_p), ("rows", c_void_p), ("out", c_void_p),
+        ("num_out", c_int), ("hidden", c_int), ("streams", c_int), ("s_in", c_int), ("planes", c_int),
+        ("y_dtype", c_int), ("out_dtype", c_int), ("plane_stride", c_long), ("eps", c_float),
     ]
 
 
@@ -223,6 +234,93 @@ class HipOps:
             c_long(plane_stride), _stream()))
         return out
 
+    def mix_norm(self, streams, update, read, weight, bias, eps, out_dtype, rows=None):
+        """The step between two sub-layers over residual streams ``[T, S, H]`` (or one stream
+        ``[T, H]``), float32, in one kernel: apply the pending ``update`` in place (a
+        ``StreamUpdate``: ``new[:, t] = sum_s mix[s, t] old[:, s] + out[t] y``; a plain tensor or
+        planes: added, one stream only; None: nothing), form ``sum_t read[t] new[:, t]`` and
+        normalise it: layer norm with ``bias``, RMS norm without. With ``rows`` only those rows are
+        normalised and nothing is written back."""
+        one = streams.dim() == 2
+        t, s, h = (streams.shape[0], 1, streams.shape[1]) if one else streams.shape
+        _need(streams, "residual streams", torch.float32)
+        _need(weight, "norm weight", torch.float32, (h,))
+        a = _MixNormArgs()
+        a.x_in, a.streams, a.s_in, a.hidden, a.eps = streams.data_ptr(), s, s, h, eps
+        a.weight, a.bias = weight.data_ptr(), _addr(None if bias is None else _need(bias, "norm bias", torch.float32, (h,)))
+        if update is not None:
+            y = update.y if hasattr(update, "y") else update
+            if hasattr(update, "y"):
+                a.mix = _need(update.mix, "stream mix", torch.float32, (s, s)).data_ptr()
+                a.out_w = _need(update.out, "stream out", torch.float32, (s,)).data_ptr()
+            elif s != 1:
+                raise OpsError("several residual streams take a StreamUpdate, not a plain delta")
+            if y.dim() == 3:
+                a.planes, a.plane_stride = y.shape[0], t * h
+                _need(y, "pending output", shape=(y.shape[0], t, h))
+            else:
+                a.planes = 1
+                _need(y, "pending output", shape=(t, h))
+            a.y, a.y_dtype = y.data_ptr(), _CODE[y.dtype]
+        if read is not None:
+            a.read = _need(read, "stream read", torch.float32, (s,)).data_ptr()
+        n_out = t
+        if rows is not None:
+            a.rows = _need(rows, "rows", torch.int32).data_ptr()
+            n_out = rows.numel()
+        elif update is not None:
+            a.x_out = streams.data_ptr()
+        out = torch.empty((n_out, h), dtype=out_dtype, device=streams.device)
+        a.out, a.out_dtype, a.num_out = out.data_ptr(), _CODE[out_dtype], n_out
+        self._check(self.lib, self.lib.qrt_mix_norm(byref(a), _stream()))
+        return out
+
+    # ---- routed experts --------------------------------------------------------------
+    def route_top(self, x, router, router_bias, top):
+        """Router logits ``x W^T + b`` in float32, the ``top`` largest per token and the softmax
+        over those alone: (int32 [T, top], float32 [T, top])."""
+        t, h = x.shape
+        _need(x, "x")
+        n = router.shape[0]
+        _need(router, "router", torch.float32, (n, h))
+        if router_bias is not None:
+            _need(router_bias, "router bias", torch.float32, (n,))
+        index = torch.empty((t, top), dtype=torch.int32, device=x.device)
+        weight = torch.empty((t, top), dtype=torch.float32, device=x.device)
+        self._check(self.lib, self.lib.qrt_route_top(_ptr(x), _CODE[x.dtype], _ptr(router), _ptr(router_bias),
+                                                     _ptr(index), _ptr(weight), c_int(t), c_int(h), c_int(n),
+                                                     c_int(top), _stream()))
+        return index, weight
+
+    def moe_swiglu(self, x, gate_up, down, index, weight):
+        """``sum_j weight[t, j] * down[e] (silu(gate[e] x) * (up[e] x))`` with ``e = index[t, j]``;
+        ``gate_up`` [E, 2I, H] (gate rows first), ``down`` [E, H, I]. float32 [T, H]."""
+        t, h = x.shape
+        n, two_i, _ = gate_up.shape
+        inter = two_i // 2
+        top = index.shape[1]
+        _need(x, "x")
+        _need(gate_up, "expert gate/up", x.dtype, (n, 2 * inter, h))
+        _need(down, "expert down", x.dtype, (n, h, inter))
+        _need(index, "expert index", torch.int32, (t, top))
+        _need(weight, "expert weight", torch.float32, (t, top))
+        act = torch.empty((t * top, inter), dtype=x.dtype, device=x.device)
+        out = torch.empty((t, h), dtype=torch.float32, device=x.device)
+        self._check(self.lib, self.lib.qrt_moe_pairs(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(index), _ptr(weight),
+                                                     _ptr(act), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
+                                                     c_int(inter), c_int(n), c_int(top), _stream()))
+        return out
+
+    def sigmoid_gate(self, out, gate):
+        """``out *= sigmoid(gate)`` in place; ``gate`` may be columns of a wider matrix."""
+        t, w = out.shape
+        _need(out, "attention output")
+        if gate.dtype != out.dtype or tuple(gate.shape) != (t, w) or gate.stride(1) != 1:
+            raise OpsError(f"gate {tuple(gate.shape)} {gate.dtype} does not fit output {tuple(out.shape)} {out.dtype}")
+        self._check(self.lib, self.lib.qrt_sigmoid_gate(_ptr(out), c_void_p(gate.data_ptr()), c_long(gate.stride(0)),
+                                                        _CODE[out.dtype], c_int(t), c_int(w), _stream()))
+        return out
+
     def swiglu(self, gate_up):
         _need(gate_up, "gate_up")
         t, two_i = gate_up.shape
@@ -387,12 +485,14 @@ class HipOps:
     rope_table_from_tokens = 256
 
     def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache, ctx=None,
-                           angles_key=None):
+                           angles_key=None, value_dim=None, extra=0):
         """Per-head RMSNorm of queries and keys, NeoX rotation, and the write of keys and values into
         the cache, in one pass over ``qkv``; returns the queries. With the step's context given,
-        the angles of a long step come from ``rope_table`` (``angles_key`` as there)."""
+        the angles of a long step come from ``rope_table`` (``angles_key`` as there). Values may
+        have ``value_dim`` elements a head; ``extra`` columns behind them are left alone."""
         t, width = qkv.shape
-        _need(qkv, "qkv", shape=(t, (nq + 2 * nkv) * d))
+        dv = d if value_dim is None else int(value_dim)
+        _need(qkv, "qkv", shape=(t, (nq + nkv) * d + nkv * dv + extra))
         for name, w in (("q_norm", q_w), ("k_norm", k_w)):
             if w is not None:
                 _need(w, name, torch.float32, (d,))
@@ -412,9 +512,10 @@ class HipOps:
             a.rope = self.rope_table(ctx, inv_freq, angles_key).data_ptr()
         a.q_out = q.data_ptr()
         a.num_tokens, a.nq, a.nkv, a.nv, a.head_dim, a.eps = t, nq, nkv, nkv, d, eps
+        a.value_dim = dv
         pages = 0
         if cache is not None:
-            pages = self._check_cache(cache, nkv, d, qkv.dtype)
+            pages = self._check_cache(cache, nkv, d, qkv.dtype, dv)
             _need(cache.group.slots, "slots", torch.int32, (t,))
             a.slots, a.k_cache, a.v_cache = _addr(cache.group.slots), _addr(cache.k), _addr(cache.v)
             a.page_size = cache.group.page_size
@@ -472,11 +573,11 @@ class HipOps:
         self._qk(a, k.dtype, pages)
 
     @staticmethod
-    def _check_cache(cache, nkv, d, dtype) -> int:
+    def _check_cache(cache, nkv, d, dtype, dv=None) -> int:
         ps = cache.group.page_size
         pages = cache.k.shape[0]
         _need(cache.k, "key cache", dtype, (pages, nkv, ps, d))
-        _need(cache.v, "value cache", dtype, (pages, nkv, d, ps))
+        _need(cache.v, "value cache", dtype, (pages, nkv, d if dv is None else dv, ps))
         return pages
 
     # ---- attention ---------------------------------------------------------------
@@ -498,10 +599,13 @@ class HipOps:
             ctx.per_pass[key] = table
         return table
 
-    def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache) -> bool:
+    def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache, value_dim=None, chunk=None, softcap=None,
+                               gate=None) -> bool:
         """Whether ``decode_attention`` serves this step: one token per sequence, bfloat16, a head
         size that keeps a rotation pair in one lane (a multiple of 64, up to 256), at most 16
         query heads per key head, and a layer that writes its own cache."""
+        if value_dim not in (None, d) or chunk is not None or softcap is not None or gate is not None:
+            return False
         return (self.fuse_decode and qkv.dtype == torch.bfloat16 and ctx.max_q_len == 1
                 and ctx.num_tokens == ctx.num_seqs and d % 64 == 0 and d <= 256 and nq // nkv <= 16
                 and cache is not None and cache.writes and cache.group.page_size % 8 == 0
@@ -535,10 +639,18 @@ class HipOps:
         self._launch_attention(None, out, cache, ctx, nq, nkv, d, scale, window or 0, None, True, own)
         return out
 
-    def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window):
+    def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window, chunk=None, softcap=None, value_dim=None,
+                        gate=None):
+        """Attention of every query over its sequence's cache. Beyond the plain form: a mask of
+        chunks instead of a window (``chunk``), a tanh cap on the scaled scores (``softcap``),
+        values of ``value_dim`` elements, and a ``gate`` [T, nq * value_dim] (columns of a wider
+        matrix will do) whose sigmoid multiplies the output."""
         t = ctx.num_tokens
+        dv = d if value_dim is None else int(value_dim)
         _need(q, "q", shape=(t, nq * d))
-        self._check_cache(cache, nkv, d, q.dtype)
+        self._check_cache(cache, nkv, d, q.dtype, dv)
+        if gate is not None and (gate.dtype != q.dtype or tuple(gate.shape) != (t, nq * dv) or gate.stride(1) != 1):
+            raise OpsError(f"gate {tuple(gate.shape)} {gate.dtype} does not fit {t} tokens of {nq} heads of {dv}")
         table = _need(cache.group.block_table, "block table", torch.int32)
         if table.shape[0] != ctx.num_seqs:
             raise OpsError(f"block table has {table.shape[0]} rows for {ctx.num_seqs} sequences")
@@ -546,9 +658,12 @@ class HipOps:
         need_pages = (ctx.max_kv_len + ps - 1) // ps
         if table.shape[1] < need_pages:
             raise OpsError(f"block table is {table.shape[1]} pages wide, the longest sequence needs {need_pages}")
-        out = torch.empty_like(q)
-        if q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
+        out = torch.empty((t, nq * dv), dtype=q.dtype, device=q.device)
+        plain = chunk is None and softcap is None and dv == d
+        if plain and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
             self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0)
+            if gate is not None:
+                self.sigmoid_gate(out, gate)
         else:
             a = _AttnArgs()
             a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
@@ -557,6 +672,9 @@ class HipOps:
             a.block_table, a.table_width = table.data_ptr(), table.shape[1]
             a.num_tokens, a.nq, a.nkv, a.head_dim, a.page_size = t, nq, nkv, d, ps
             a.window, a.scale = window or 0, scale
+            a.chunk, a.softcap, a.value_dim = chunk or 0, softcap or 0.0, dv
+            if gate is not None:
+                a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
             self._check(self.lib, self.lib.qrt_attention_f32(byref(a), _CODE[q.dtype], _stream()))
         return out
 
