@@ -23,7 +23,9 @@
 // Softmax is online, float32, in base 2 (scale * log2 e is folded into the
 // exponent's argument); probabilities are rounded to bfloat16 for the second
 // product, accumulation is float32. Key j is visible to the row at position p
-// iff j <= p and (no window or j > p - window).
+// iff first_seen(p) <= j <= p: the first key a row sees is 0, or p - window + 1 with a window, or
+// the first position of p's chunk (p - p % chunk) with a mask of chunks. With a score cap the
+// scaled scores become cap * tanh(score / cap) before the softmax.
 #include "common.h"
 #include <math.h>
 
@@ -88,7 +90,28 @@ struct AttnTileArgs {
   // the compute units. qrt_attention_work_list fills the list from the step's lengths.
   int split_blocks, max_items;
   int* items;              // [max_items][2] or null
+  int chunk;               // > 0: a query sees the keys of its own chunk of this many positions (no window then)
+  float cap_in, cap_out;   // score cap c > 0: cap_in = scale / c, cap_out = c / scale; 0: no cap
 };
+
+// The first key position that the query at position p sees. It does not fall as p grows, so for a
+// range of positions the lowest first key is that of the lowest position, the highest that of the
+// highest. With a window it may be negative.
+__device__ __forceinline__ int first_seen(int p, int window, int chunk) {
+  return window > 0 ? p - window + 1 : (chunk > 0 ? p - p % chunk : 0);
+}
+
+// Scores (raw dot products) under a cap: s -> tanh(s * cap_in) * cap_out, so that the scaling that
+// follows yields cap * tanh(scaled score / cap). tanh x = 1 - 2 / (1 + e^(2x)) from one
+// exponential and one reciprocal; both ends saturate to +-1 (e^(2x) -> inf or 0).
+__device__ __forceinline__ void cap_scores(f32x4_t sc[2], float cap_in, float cap_out) {
+  const float k = cap_in * 2.885390081777927f;  // 2 log2 e
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float ex = __builtin_amdgcn_exp2f(sc[e >> 2][e & 3] * k);
+    sc[e >> 2][e & 3] = fmaf(-2.0f * cap_out, __builtin_amdgcn_rcpf(1.0f + ex), cap_out);
+  }
+}
 
 constexpr int D = QRT_HEAD_DIM;
 constexpr int KFULL = D / 32;        // 32-wide steps of the first product
@@ -137,16 +160,17 @@ __device__ __forceinline__ float row_max4(float x) {
 }
 
 __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t* vv, bool masked, int base,
-                                            int quad, bool row_valid, int qpos, int window, float scale_log2,
-                                            float& m, float& l, f32x4_t* o) {
+                                            int quad, bool row_valid, int qpos, int window, int chunk,
+                                            float scale_log2, float& m, float& l, f32x4_t* o) {
   float s[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) s[e] = sc[e >> 2][e & 3];
   if (masked) {  // the same for the whole wave
+    const int lo_row = first_seen(qpos, window, chunk);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int key = base + 8 * quad + e;
-      const bool vis = row_valid && key <= qpos && (window == 0 || key > qpos - window);
+      const bool vis = row_valid && key <= qpos && key >= lo_row;
       s[e] = vis ? s[e] : -INFINITY;
     }
   }
@@ -183,7 +207,7 @@ __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t*
 // the exponentials of one tile can issue while the matrix pipe works on another's products.
 template <int RT>
 __device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x8_t* vv, unsigned whole, int base,
-                                             int quad, const bool* row_valid, const int* qpos, int window,
+                                             int quad, const bool* row_valid, const int* qpos, int window, int chunk,
                                              float scale_log2, float* m, float* l, f32x4_t (*o)[DB]) {
   // whole: bit t says that every row of tile t sees all 32 keys (one scalar for the wave: an
   // array of flags went through vector registers, a dozen instructions per block of keys)
@@ -194,13 +218,15 @@ __device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x
     for (int e = 0; e < 8; ++e) s[t][e] = sc[t][e >> 2][e & 3];
   if (whole != (1u << RT) - 1) {  // the same for the whole wave
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
+    for (int t = 0; t < RT; ++t) {
+      const int lo_row = first_seen(qpos[t], window, chunk);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = base + 8 * quad + e;
-        const bool vis = ((whole >> t) & 1) || (row_valid[t] && key <= qpos[t] && (window == 0 || key > qpos[t] - window));
+        const bool vis = ((whole >> t) & 1) || (row_valid[t] && key <= qpos[t] && key >= lo_row);
         s[t][e] = vis ? s[t][e] : -INFINITY;
       }
+    }
   }
   float m_use[RT], corr[RT];
   bool moved = false;
@@ -316,7 +342,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
 
   // per tile: this lane's row, its token's position, and Q as B operands kept for the whole loop
   bool row_valid[RT];
-  int qpos[RT], tile_pos_min[RT], tile_pos_max[RT];  // this lane's position; the tile's range of positions
+  int qpos[RT], tile_pos_min[RT], tile_lo_max[RT];  // this lane's position; the tile's lowest position, and the
+                                                     // first key that its highest position sees
   size_t row_index[RT];
   bf16x8_t qreg[RT][KFULL > 0 ? KFULL : 1];
   bf16x8_t qtail[RT];
@@ -329,7 +356,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
     qpos[t] = first_pos + tok;
     // the same for every lane: kept in scalar registers so that the choice below is a plain branch
     tile_pos_min[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t, n_rows - 1) / g);
-    tile_pos_max[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t + 15, n_rows - 1) / g);
+    tile_lo_max[t] = __builtin_amdgcn_readfirstlane(
+        first_seen(first_pos + min(row0 + 16 * t + 15, n_rows - 1) / g, a.window, a.chunk));
     row_index[t] = (size_t)(q_begin + tok) * a.nq + kvh * g + hg;
     const bf16_t* qp = a.q + row_index[t] * D;
 #pragma unroll
@@ -341,7 +369,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
   // keys this wave may need: [lo, pos_max]
   const int row_last = min(row0 + 16 * RT - 1, n_rows - 1);
   const int pos_min = first_pos + row0 / g, pos_max = first_pos + row_last / g;
-  const int lo = a.window > 0 ? max(0, pos_min - a.window + 1) : 0;
+  const int lo = max(0, first_seen(pos_min, a.window, a.chunk));
   const int blk_begin = lo >> 5, blk_end = (pos_max >> 5) + 1;
   const int per = (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
   const int b0 = blk_begin + split * per;
@@ -387,9 +415,11 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
           if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kt[kb], qtail[t], acc, 0, 0, 0);
           s[kb] = acc;
         }
-        // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
-        const bool whole = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
-        tile_update(s, blk.v, !whole, base, quad, row_valid[t], qpos[t], a.window, a.scale_log2, m[t], l[t], o[t]);
+        if (a.cap_in > 0.f) cap_scores(s, a.cap_in, a.cap_out);
+        // every row of the tile sees the whole block unless it touches the diagonal or the edge of
+        // a window or a chunk
+        const bool whole = base + 31 <= tile_pos_min[t] && base >= tile_lo_max[t];
+        tile_update(s, blk.v, !whole, base, quad, row_valid[t], qpos[t], a.window, a.chunk, a.scale_log2, m[t], l[t], o[t]);
       }
 #pragma unroll
       for (int i = 0; i < 3; ++i) pg[i] = pg_next[i];
@@ -449,11 +479,13 @@ constexpr int KROW = D % 32 == 0 ? D + 16 : D;  // elements per key row in LDS
 // maximum and the accumulator shrunk as in tiles_update.
 constexpr float LAZY = 8.0f;
 
-__device__ __forceinline__ void tile_mask(f32x4_t sc[2], int base, int quad, bool row_valid, int qpos, int window) {
+__device__ __forceinline__ void tile_mask(f32x4_t sc[2], int base, int quad, bool row_valid, int qpos, int window,
+                                          int chunk) {
+  const int lo_row = first_seen(qpos, window, chunk);
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int key = base + 8 * quad + e;
-    const bool vis = row_valid && key <= qpos && (window == 0 || key > qpos - window);
+    const bool vis = row_valid && key <= qpos && key >= lo_row;
     sc[e >> 2][e & 3] = vis ? sc[e >> 2][e & 3] : -INFINITY;
   }
 }
@@ -525,7 +557,8 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
   const int* table = a.block_table + (size_t)seq * a.table_width;
 
   bool row_valid[RT];
-  int qpos[RT], tile_pos_min[RT], tile_pos_max[RT];  // this lane's position; the tile's range of positions
+  int qpos[RT], tile_pos_min[RT], tile_lo_max[RT];  // this lane's position; the tile's lowest position, and the
+                                                     // first key that its highest position sees
   size_t row_index[RT];
   bf16x8_t qreg[RT][KFULL > 0 ? KFULL : 1];
   bf16x8_t qtail[RT];
@@ -538,7 +571,8 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
     qpos[t] = first_pos + tok;
     // the same for every lane: kept in scalar registers so that the choice below is a plain branch
     tile_pos_min[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t, n_rows - 1) / g);
-    tile_pos_max[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t + 15, n_rows - 1) / g);
+    tile_lo_max[t] = __builtin_amdgcn_readfirstlane(
+        first_seen(first_pos + min(row0 + 16 * t + 15, n_rows - 1) / g, a.window, a.chunk));
     row_index[t] = (size_t)(q_begin + tok) * a.nq + kvh * g + hg;
     const bf16_t* qp = a.q + row_index[t] * D;
 #pragma unroll
@@ -550,7 +584,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
   // keys the block of waves needs, and the part of them this wave needs
   const int blk_last_row = min(tile_row0 + 64 * RT - 1, n_rows - 1);
   const int blk_pos_min = first_pos + tile_row0 / g, blk_pos_max = first_pos + blk_last_row / g;
-  const int lo = a.window > 0 ? max(0, blk_pos_min - a.window + 1) : 0;
+  const int lo = max(0, first_seen(blk_pos_min, a.window, a.chunk));
   // the blocks of keys of this block of waves, and of them the part of this split
   const int all_b0 = lo >> 5, all_b1 = (blk_pos_max >> 5) + 1;
   const int per = (all_b1 - all_b0 + a.num_splits - 1) / a.num_splits;
@@ -559,7 +593,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
   if (wave_has_rows) {
     const int row_last = min(row0 + 16 * RT - 1, n_rows - 1);
     const int pos_min = first_pos + row0 / g, pos_max = first_pos + row_last / g;
-    wb0 = (a.window > 0 ? max(0, pos_min - a.window + 1) : 0) >> 5;
+    wb0 = max(0, first_seen(pos_min, a.window, a.chunk)) >> 5;
     wb1 = min((pos_max >> 5) + 1, b1);  // not into the next split's blocks
   }
 
@@ -673,11 +707,11 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
           if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[s2], qtail[t], acc, 0, 0, 0);
           sc[s2] = acc;
         }
+        if (a.cap_in > 0.f) cap_scores(sc, a.cap_in, a.cap_out);  // the same for the whole launch
       };
-      // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
-      auto sees_all = [&](int t) {
-        return (base + 31 <= tile_pos_min[t]) & ((a.window == 0) | (base > tile_pos_max[t] - a.window));
-      };
+      // every row of the tile sees the whole block unless it touches the diagonal or the edge of a
+      // window or a chunk
+      auto sees_all = [&](int t) { return (base + 31 <= tile_pos_min[t]) & (base >= tile_lo_max[t]); };
       if constexpr (RT == 2) {
         f32x4_t sc0[2], sc1[2];
         bf16x8_t pb0, pb1;
@@ -688,11 +722,11 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
         const bool jumps = mx0 * a.scale_log2 > m[0] + LAZY || mx1 * a.scale_log2 > m[1] + LAZY;
         if (edge || __any(jumps)) {
           if (!sees_all(0)) {
-            tile_mask(sc0, base, quad, row_valid[0], qpos[0], a.window);
+            tile_mask(sc0, base, quad, row_valid[0], qpos[0], a.window, a.chunk);
             mx0 = lane_max(sc0);
           }
           if (!sees_all(1)) {
-            tile_mask(sc1, base, quad, row_valid[1], qpos[1], a.window);
+            tile_mask(sc1, base, quad, row_valid[1], qpos[1], a.window, a.chunk);
             mx1 = lane_max(sc1);
           }
           tile_move_reference(mx0, a.scale_log2, m[0], l[0], o[0]);
@@ -712,7 +746,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
           scores(t, sc[t]);
           whole |= (unsigned)sees_all(t) << t;
         }
-        tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+        tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.chunk, a.scale_log2, m, l, o);
       }
     }
   };
@@ -888,11 +922,12 @@ constexpr int DW = 4;
 
 // The 32-key blocks of the cache that a tile of the decode kernel walks: [begin, end). `fused`:
 // the cache holds the keys before the tile's one token (which the kernel adds from registers).
-__device__ __forceinline__ void decode_key_blocks(int kv_len, int q_len, int window, bool fused, int& begin, int& end) {
+__device__ __forceinline__ void decode_key_blocks(int kv_len, int q_len, int window, int chunk, bool fused, int& begin,
+                                                  int& end) {
   const int own = fused ? 1 : 0;
   const int first_pos = kv_len - q_len;
   const int pos_max = first_pos + max(q_len, 1) - 1 - own;
-  const int lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+  const int lo = max(0, first_seen(first_pos, window, chunk));
   const bool any_cached = !fused || (pos_max >= lo && window != 1);
   begin = lo >> 5;
   end = any_cached ? (pos_max >> 5) + 1 : begin;
@@ -907,7 +942,7 @@ __global__ __launch_bounds__(256) void attention_work_list_kernel(AttnTileArgs a
   for (int t = threadIdx.x; t < a.num_tiles; t += blockDim.x) {
     const int seq = a.tile_seq ? a.tile_seq[t] : t;
     int begin, end;
-    decode_key_blocks(a.kv_lens[seq], a.cu_q[seq + 1] - a.cu_q[seq], a.window, fused != 0, begin, end);
+    decode_key_blocks(a.kv_lens[seq], a.cu_q[seq + 1] - a.cu_q[seq], a.window, a.chunk, fused != 0, begin, end);
     const int blocks = end - begin;
     whole[t] = blocks / a.split_blocks;
     rest[t] = blocks % a.split_blocks != 0 || blocks == 0 ? 1 : 0;
@@ -935,7 +970,8 @@ __global__ __launch_bounds__(256) void attention_work_list_kernel(AttnTileArgs a
 
 __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg, bf16x8_t qtail, int base, int lo,
                                               int pos_min, int pos_max, int quad, bool row_valid, int qpos,
-                                              int window, float scale_log2, float& m, float& l, f32x4_t* o) {
+                                              int window, int chunk, float cap_in, float cap_out, float scale_log2,
+                                              float& m, float& l, f32x4_t* o) {
   f32x4_t s[2];
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
@@ -945,8 +981,9 @@ __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg
     if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kt[kb], qtail, acc, 0, 0, 0);
     s[kb] = acc;
   }
+  if (cap_in > 0.f) cap_scores(s, cap_in, cap_out);
   // the same for the whole wave: does every row see all 32 keys?
-  const bool whole = base + 31 <= pos_min && (window == 0 || base > pos_max - window);
+  const bool whole = base + 31 <= pos_min && base >= first_seen(pos_max, window, chunk);
   if (!whole) {
     // values of keys outside [lo, pos_max] came from a clamped place, or from places after the
     // sequence's last key in its last page, and may be anything
@@ -955,7 +992,7 @@ __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg
 #pragma unroll
     for (int i = 0; i < DB; ++i) blk.v[i] = keep_first(blk.v[i], keep);
   }
-  tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, scale_log2, m, l, o);
+  tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, chunk, scale_log2, m, l, o);
 }
 
 // One head of a token's product (x, D elements, D a multiple of 64) as an MFMA operand: RMSNorm
@@ -1057,9 +1094,9 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
   const int window = FUSED && a.window > 0 ? a.window - 1 : a.window;
   const int qpos_c = qpos - own;
   const int pos_min = first_pos - own, pos_max = first_pos + (max(n_rows, 1) - 1) / g - own;
-  const int lo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
+  const int lo = max(0, first_seen(first_pos, a.window, a.chunk));
   int blk_begin, blk_end;
-  decode_key_blocks(kv_len, q_len, a.window, FUSED, blk_begin, blk_end);
+  decode_key_blocks(kv_len, q_len, a.window, a.chunk, FUSED, blk_begin, blk_end);
   // equal parts of the sequence's blocks, or pieces of a fixed length, as many as it has
   const int per = a.items ? a.split_blocks : (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
   const int last_split = a.items ? max(1, (blk_end - blk_begin + per - 1) / per) - 1 : (int)gridDim.z - 1;
@@ -1103,6 +1140,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
         sc[1] = sc[0];
 #pragma unroll
         for (int i = 0; i < KFULL; ++i) sc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[i], qreg[i], sc[0], 0, 0, 0);
+        if (a.cap_in > 0.f) cap_scores(sc, a.cap_in, a.cap_out);
         bf16x8_t vv[DB];
 #pragma unroll
         for (int i = 0; i < DB; ++i) {
@@ -1110,7 +1148,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
           for (int e = 0; e < 8; ++e) vv[i][e] = (bf16_t)0.0f;
           if (quad == 0) vv[i][0] = vraw[16 * i + r16];
         }
-        tile_update(sc, vv, true, first_pos, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+        tile_update(sc, vv, true, first_pos, quad, row_valid, qpos, a.window, a.chunk, a.scale_log2, m, l, o);
       }
     }
   };
@@ -1137,12 +1175,12 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     block_pages<P2>(table, min(b + 3 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
     if (FUSED) own_token();  // while the first keys and values are on their way
     while (true) {
-      block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.scale_log2, m, l, o);
+      block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.chunk, a.cap_in, a.cap_out, a.scale_log2, m, l, o);
       block_load<P2, DECODE_ONCE>(a, kvh, min(b + 2 * DW, last) << 5, lo, pos_max, r16, quad, pgA, A, b + 2 * DW <= last);
       block_pages<P2>(table, min(b + 4 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
       b += DW;
       if (b >= b1) break;
-      block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.scale_log2, m, l, o);
+      block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.chunk, a.cap_in, a.cap_out, a.scale_log2, m, l, o);
       block_load<P2, DECODE_ONCE>(a, kvh, min(b + 2 * DW, last) << 5, lo, pos_max, r16, quad, pgB, B, b + 2 * DW <= last);
       block_pages<P2>(table, min(b + 4 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
       b += DW;
@@ -1229,6 +1267,8 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   QRT_CHECK(a.num_splits >= 1 && a.num_splits <= 65535 && a.nkv <= 65535, "attention: bad split or head count");
   QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
+  QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a mask of chunks, not both");
+  QRT_CHECK((a.cap_in > 0.f) == (a.cap_out > 0.f), "attention: a score cap needs both of its factors");
   QRT_CHECK(a.items ? a.split_blocks > 0 && a.max_items >= a.num_tiles && a.max_items <= 65535
                     : a.split_blocks == 0,
             "attention (decode): pieces of %d blocks with a list of %d items for %d sequences", a.split_blocks,
@@ -1295,6 +1335,8 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   QRT_CHECK(a.num_splits >= 1 && a.num_splits <= 65535 && a.nkv <= 65535, "attention: bad split or head count");
   QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
+  QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a mask of chunks, not both");
+  QRT_CHECK((a.cap_in > 0.f) == (a.cap_out > 0.f), "attention: a score cap needs both of its factors");
   if (a.num_tiles == 0) return 0;
   const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   QRT_CHECK((long long)a.num_tiles * a.nkv < (1ll << 31), "attention: %d tiles x %d key heads is too many blocks", a.num_tiles, a.nkv);

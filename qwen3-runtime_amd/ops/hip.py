@@ -79,6 +79,7 @@ class _AttnTileArgs(Structure):
         ("qkv", c_void_p), ("qkv_stride", c_long), ("q_weight", c_void_p), ("k_weight", c_void_p),
         ("rope", c_void_p), ("slots", c_void_p), ("eps", c_float), ("split_blocks", c_int),
         ("max_items", c_int), ("items", c_void_p),
+        ("chunk", c_int), ("cap_in", c_float), ("cap_out", c_float),
     ]
 
 
@@ -604,7 +605,7 @@ class HipOps:
         """Whether ``decode_attention`` serves this step: one token per sequence, bfloat16, a head
         size that keeps a rotation pair in one lane (a multiple of 64, up to 256), at most 16
         query heads per key head, and a layer that writes its own cache."""
-        if value_dim not in (None, d) or chunk is not None or softcap is not None or gate is not None:
+        if value_dim not in (None, d):
             return False
         return (self.fuse_decode and qkv.dtype == torch.bfloat16 and ctx.max_q_len == 1
                 and ctx.num_tokens == ctx.num_seqs and d % 64 == 0 and d <= 256 and nq // nkv <= 16
@@ -612,14 +613,15 @@ class HipOps:
                 and cache.k.dtype == torch.bfloat16)
 
     def decode_attention(self, qkv, cache, ctx, nq, nkv, d, scale, window, q_w, k_w, eps, inv_freq,
-                         angles_key=None):
+                         angles_key=None, chunk=None, softcap=None, gate=None, value_dim=None):
         """``paged_attention(qk_norm_rope_store(qkv, ...))`` for a step of single tokens, in one
         kernel: each block forms its queries from ``qkv`` (RMSNorm per head, NeoX rotation by the
         step's angle table), attends over the cached keys before the token, adds the token's own
         key and value from registers and stores them into the cache for later steps. Saves the
         kernel between the product and the attention, and the round trip of the queries."""
         t, width = qkv.shape
-        _need(qkv, "qkv", torch.bfloat16, (t, (nq + 2 * nkv) * d))
+        extra = 0 if gate is None else gate.shape[1]  # the gate's columns, behind q | k | v
+        _need(qkv, "qkv", torch.bfloat16, (t, (nq + 2 * nkv) * d + extra))
         self._check_cache(cache, nkv, d, qkv.dtype)
         for name, w in (("q_norm", q_w), ("k_norm", k_w)):
             if w is not None:
@@ -636,7 +638,10 @@ class HipOps:
         own = {"qkv": qkv, "q_weight": q_w, "k_weight": k_w, "eps": eps,
                "rope": None if inv_freq is None else self.rope_table(ctx, inv_freq, angles_key)}
         out = torch.empty((t, nq * d), dtype=qkv.dtype, device=qkv.device)
-        self._launch_attention(None, out, cache, ctx, nq, nkv, d, scale, window or 0, None, True, own)
+        self._launch_attention(None, out, cache, ctx, nq, nkv, d, scale, window or 0, None, True, own,
+                               chunk=chunk or 0, softcap=softcap or 0.0)
+        if gate is not None:
+            self.sigmoid_gate(out, gate)
         return out
 
     def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window, chunk=None, softcap=None, value_dim=None,
@@ -659,9 +664,8 @@ class HipOps:
         if table.shape[1] < need_pages:
             raise OpsError(f"block table is {table.shape[1]} pages wide, the longest sequence needs {need_pages}")
         out = torch.empty((t, nq * dv), dtype=q.dtype, device=q.device)
-        plain = chunk is None and softcap is None and dv == d
-        if plain and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
-            self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0)
+        if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
+            self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0, chunk or 0, softcap or 0.0)
             if gate is not None:
                 self.sigmoid_gate(out, gate)
         else:
@@ -799,7 +803,7 @@ class HipOps:
     # mixed steps: sequences with few rows leave the prompt kernel when their context is this long
     split_launch_min_kv = 1024
 
-    def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window):
+    def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window, chunk=0, softcap=0.0):
         """Which kernel for which sequences. Steps of decoded tokens only: the decode kernel.
         Other steps: the prompt kernels; but sequences of at most 16 rows with a long context
         (decoded tokens beside a prompt portion) would each walk all their keys in one block
@@ -810,22 +814,26 @@ class HipOps:
         g = nq // nkv
         seqs = range(ctx.num_seqs)
         if ctx.max_q_len * g <= 16 and d <= 256:
-            return self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, True)
+            return self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, True, chunk=chunk, softcap=softcap)
         small = [s for s in seqs if ctx.q_lens_host[s] * g <= 16]
         if (d <= 256 and small and len(small) < ctx.num_seqs
                 and max(ctx.kv_lens_host[s] for s in small) >= self.split_launch_min_kv):
             small_set = set(small)
             big = [s for s in seqs if s not in small_set]
-            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, small, True)
-            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, big, False)
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, small, True, chunk=chunk, softcap=softcap)
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, big, False, chunk=chunk, softcap=softcap)
             return
-        self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False)
+        self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False, chunk=chunk, softcap=softcap)
 
-    def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode, own=None):
+    def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode, own=None,
+                          chunk=0, softcap=0.0):
         """One launch over the sequences in ``subset`` (None: all of the step's). ``own``: the
         decode kernel takes the tokens' queries, own keys and own values from the q/k/v product
-        (``decode_attention``); ``q`` is then None."""
+        (``decode_attention``); ``q`` is then None. ``chunk``: a mask of chunks in place of a
+        window; ``softcap``: the cap on the scaled scores."""
         lib = attention_library(d)
+        # how far back a query can see at most: what the choices below (key splits, pieces) go by
+        reach = window or chunk
         g = nq // nkv
         if subset is None:  # the step's own maxima: under a graph they are those of its bucket
             q_lens, kv_lens = ctx.q_lens_host, ctx.kv_lens_host
@@ -834,12 +842,13 @@ class HipOps:
             q_lens = [ctx.q_lens_host[s] for s in subset]
             kv_lens = [ctx.kv_lens_host[s] for s in subset]
             max_rows, max_kv = max(q_lens) * g, max(kv_lens)
+        seen_kv = min(max_kv, reach) if reach else max_kv  # keys that the splits divide
         waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
         # long portions: several row tiles per wave, so that loaded keys and values serve more rows
         row_tiles = 1 if max_rows <= 64 else (self.prefill_row_tiles if d <= 128 else min(2, self.prefill_row_tiles))
         # the list depends on the rows a tile holds (head geometry and kernel choice): layers of
         # another geometry in the same step get a list of their own
-        key = ("attn_plan", g, nkv, d, waves, row_tiles, decode, None if subset is None else tuple(subset))
+        key = ("attn_plan", g, nkv, d, waves, row_tiles, decode, None if subset is None else tuple(subset), reach)
         plan = ctx.scratch.get(key)
         if plan is None:  # the same for every layer of the step
             dev = out.device
@@ -848,7 +857,7 @@ class HipOps:
                 n_tiles = len(q_lens)
             else:
                 lds = waves == 4 and row_tiles >= 2 and self.prefill_through_lds
-                groups = self.choose_key_groups(q_lens, kv_lens, g, nkv, window,
+                groups = self.choose_key_groups(q_lens, kv_lens, g, nkv, reach,
                                                 ctx.scratch.get("attn_splits")) if lds else 0
                 host, n_tiles = self.plan_tiles(q_lens, kv_lens, g, 16 * waves * row_tiles, nkv,
                                                 self.resident_blocks if waves == 4 and row_tiles >= 2 and groups < 2
@@ -863,23 +872,27 @@ class HipOps:
             ctx.scratch[key] = plan
         tiles, n_tiles, tokens, groups = plan
         splits = ctx.scratch.get("attn_splits") or (
-            self.choose_decode_splits(n_tiles, nkv, max_kv) if decode else self.choose_splits(n_tiles, nkv, max_kv))
+            self.choose_decode_splits(n_tiles, nkv, seen_kv) if decode else self.choose_splits(n_tiles, nkv, seen_kv))
         a = _AttnTileArgs()
+        a.chunk = chunk
+        if softcap:
+            a.cap_in, a.cap_out = scale / softcap, softcap / scale
         piece = None
         if decode and n_tiles <= 1024:
             piece = ctx.scratch.get("attn_piece")  # keys per piece, a multiple of 32: asked for outright
             if piece is None and "attn_splits" not in ctx.scratch:
                 # the lengths as they are; a capture sees its bucket's instead and is told them beside
-                piece = self.choose_decode_piece(ctx.scratch.get("attn_lens") or kv_lens, nkv)
+                lens = ctx.scratch.get("attn_lens") or kv_lens
+                piece = self.choose_decode_piece([min(n, reach) for n in lens] if reach else lens, nkv)
         if piece:
             a.split_blocks = piece // 32
             # 32-key blocks a sequence of this launch can have: all its keys, or those of its
             # window, which may begin and end inside a block
-            span = (max_kv + 31) // 32 if not window else (min(max_kv, window + 32) + 31) // 32 + 1
+            span = (max_kv + 31) // 32 if not reach else (min(max_kv, reach + 32) + 31) // 32 + 1
             splits = max(1, -(-span // a.split_blocks))
             if n_tiles * splits > 65535:
                 piece, a.split_blocks = None, 0
-                splits = self.choose_decode_splits(n_tiles, nkv, max_kv)
+                splits = self.choose_decode_splits(n_tiles, nkv, seen_kv)
         a.out, a.k_cache, a.v_cache = out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
         if own is None:
             a.q = q.data_ptr()
@@ -907,7 +920,7 @@ class HipOps:
         if piece:
             # the list of (sequence, piece): from the step's lengths on the device, once per pass
             a.max_items = n_tiles * splits
-            list_key = ("attn_items", key, window, own is not None, piece, a.max_items)
+            list_key = ("attn_items", key, window, chunk, own is not None, piece, a.max_items)
             items = ctx.per_pass.get(list_key)
             if items is None:
                 items = torch.empty((a.max_items, 2), dtype=torch.int32, device=out.device)

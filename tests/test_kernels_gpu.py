@@ -823,7 +823,7 @@ def test_mixed_steps_go_through_two_launches_and_agree(ops, seqs, nq, nkv, d, ps
                              ps, nq, nkv, d, 0.125, window)
     launches = []
     inner = ops._launch_attention
-    monkeypatch.setattr(ops, "_launch_attention", lambda *a: (launches.append(a[-2:]), inner(*a))[1])
+    monkeypatch.setattr(ops, "_launch_attention", lambda *a, **kw: (launches.append(a[-2:]), inner(*a, **kw))[1])
     for min_kv, want_launches in ((1, 2), (1 << 30, 1)):
         monkeypatch.setattr(ops, "split_launch_min_kv", min_kv)
         for splits in (None, 1, 2, 5):

@@ -163,7 +163,7 @@ def test_long_context_decode_beside_a_prompt_portion(sized, monkeypatch):
     launches = []
     inner = HipOps._launch_attention
     monkeypatch.setattr(HipOps, "_launch_attention",
-                        lambda self, *a: (launches.append(a[-2:]), inner(self, *a))[1])
+                        lambda self, *a, **kw: (launches.append(a[-2:]), inner(self, *a, **kw))[1])
     got = traces.replay(load_sized(folder, steps, "bfloat16"), steps)
     assert ([0], True) in launches and ([1], False) in launches, "the mixed steps ran as two launches"
     check_rounding_noise(got, {k: want[k] for k in got})
