@@ -22,6 +22,12 @@ the live requests) over its time, against the published HBM peak, with the
 bandwidth and the MFMA rate this device delivered in a microbenchmark beside
 the published figures (``measured_peak``).
 
+Other models: ``--preset NAME`` runs the same workload on any registered configuration, so two
+designs are measured beside each other at equal sizes: ``--preset deginex_4b`` (hyper-connections,
+chunked capped gated attention, dense feed-forwards) and ``--preset deginex_4b_moe`` (every other
+feed-forward a mixture of 16 experts, 2 a token) have the widths, heads, layers and vocabulary of
+``qwen3_4b``.
+
 Other workloads: ``--workload mix`` (continuous batching of ``--requests``
 requests with prompts of 128 to 4,096 tokens, portions of 2,048, 256 outputs
 each) and any closed batch by ``--preset/--batch/--prompt-len/--context``.
@@ -151,7 +157,10 @@ def main() -> int:
     raw_full = preset_config(args.preset)
     raw = dict(raw_full)
     if args.layers is not None:
-        raw["num_hidden_layers"] = args.layers
+        if isinstance(raw.get("layers"), list):  # a configuration that lists its layers
+            raw["layers"] = raw["layers"][: args.layers]
+        else:
+            raw["num_hidden_layers"] = args.layers
     steps, warmup, trials = args.steps, args.warmup, max(1, args.trials)
     page = 16
     max_batch = args.batch if (args.no_points or args.prefill_only) else max(args.batch, 64)

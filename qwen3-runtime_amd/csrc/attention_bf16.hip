@@ -92,6 +92,11 @@ struct AttnTileArgs {
   int* items;              // [max_items][2] or null
   int chunk;               // > 0: a query sees the keys of its own chunk of this many positions (no window then)
   float cap_in, cap_out;   // score cap c > 0: cap_in = scale / c, cap_out = c / scale; 0: no cap
+  // An output gate: the result at (token, head, element) is multiplied by the sigmoid of
+  // gate[token * gate_stride + head * D + element] (the gate's columns of the product that made
+  // q, k and v, say). Applied where the output is written: here, or in the merge of key splits.
+  const bf16_t* gate;
+  long gate_stride;
 };
 
 // The first key position that the query at position p sees. It does not fall as p grows, so for a
@@ -117,6 +122,15 @@ constexpr int D = QRT_HEAD_DIM;
 constexpr int KFULL = D / 32;        // 32-wide steps of the first product
 constexpr bool KTAIL = (D % 32) != 0;  // one 16-wide step more
 constexpr int DB = D / 16;           // 16-wide blocks of the head dimension
+
+// sigmoid of the gate's element for output row `row` (= token * nq + head) and head element d; 1 without a gate
+__device__ __forceinline__ float gate_factor(const bf16_t* __restrict__ gate, long gate_stride, int nq, size_t row, int d) {
+  if (!gate) return 1.0f;
+  const size_t token = row / nq;
+  const float x = (float)gate[token * gate_stride + (row - token * nq) * D + d];
+  return 1.0f / (1.0f + __expf(-x));
+}
+
 
 // One tile of 16 rows meets one block of 32 keys: sc holds the raw scores (this lane: its row,
 // keys base + 8 quad + e), vv the block's values as MFMA operands. Online softmax in base 2;
@@ -439,7 +453,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
       for (int i = 0; i < DB; ++i) {
         bf16x4_t w;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[t][i][r] * inv);
+        for (int r = 0; r < 4; ++r)
+          w[r] = (bf16_t)(o[t][i][r] * inv * gate_factor(a.gate, a.gate_stride, a.nq, row_index[t], 16 * i + 4 * quad + r));
         *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
       }
     } else {
@@ -822,7 +837,8 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
       for (int i = 0; i < DB; ++i) {
         bf16x4_t w;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[t][i][r] * inv);
+        for (int r = 0; r < 4; ++r)
+          w[r] = (bf16_t)(o[t][i][r] * inv * gate_factor(a.gate, a.gate_stride, a.nq, row_index[t], 16 * i + 4 * quad + r));
         *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
       }
     } else {
@@ -842,9 +858,11 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefil
 // A thread takes elements threadIdx.x and threadIdx.x + blockDim.x of the row.
 template <int MAX>
 __device__ __forceinline__ void merge_few(const float* __restrict__ part_o, const float* __restrict__ lse,
-                                          bf16_t* __restrict__ out, int num_splits, size_t row) {
+                                          bf16_t* __restrict__ out, int num_splits, size_t row,
+                                          const bf16_t* __restrict__ gate, long gate_stride, int nq) {
   float ls[MAX], pv[2][MAX];
   const int d0 = min((int)threadIdx.x, D - 1), d1 = min((int)(threadIdx.x + blockDim.x), D - 1);
+  const float g0 = gate_factor(gate, gate_stride, nq, row, d0), g1 = gate_factor(gate, gate_stride, nq, row, d1);
 #pragma unroll
   for (int s = 0; s < MAX; ++s) {
     const int sc = min(s, num_splits - 1);
@@ -869,23 +887,23 @@ __device__ __forceinline__ void merge_few(const float* __restrict__ part_o, cons
       }
     }
   }
-  if ((int)threadIdx.x < D) out[row * D + threadIdx.x] = (bf16_t)(wsum > 0.f ? acc[0] / wsum : 0.f);
+  if ((int)threadIdx.x < D) out[row * D + threadIdx.x] = (bf16_t)(wsum > 0.f ? acc[0] / wsum * g0 : 0.f);
   if ((int)(threadIdx.x + blockDim.x) < D)
-    out[row * D + threadIdx.x + blockDim.x] = (bf16_t)(wsum > 0.f ? acc[1] / wsum : 0.f);
+    out[row * D + threadIdx.x + blockDim.x] = (bf16_t)(wsum > 0.f ? acc[1] / wsum * g1 : 0.f);
 }
 
 // out[row] = sum_s 2^(lse_s - M) O_s / sum_s 2^(lse_s - M); empty splits weigh 0
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
                                        bf16_t* __restrict__ out, int num_splits, const int* __restrict__ tokens,
-                                       int nq) {
+                                       int nq, const bf16_t* __restrict__ gate, long gate_stride) {
   // rows are (token, query head); with a token list the grid walks the listed tokens' rows only
   const size_t row = tokens ? (size_t)tokens[blockIdx.x / nq] * nq + blockIdx.x % nq : blockIdx.x;
   const float* lse = part_lse + row * num_splits;
   if (num_splits <= 64 && D <= 2 * (int)blockDim.x) {
-    if (num_splits <= 8) merge_few<8>(part_o, lse, out, num_splits, row);
-    else if (num_splits <= 16) merge_few<16>(part_o, lse, out, num_splits, row);
-    else if (num_splits <= 32) merge_few<32>(part_o, lse, out, num_splits, row);
-    else merge_few<64>(part_o, lse, out, num_splits, row);
+    if (num_splits <= 8) merge_few<8>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
+    else if (num_splits <= 16) merge_few<16>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
+    else if (num_splits <= 32) merge_few<32>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
+    else merge_few<64>(part_o, lse, out, num_splits, row, gate, gate_stride, nq);
     return;
   }
   float mx = -INFINITY;
@@ -901,7 +919,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
         if (w > 0.f) acc += w * po[(size_t)s * D];
       }
     }
-    out[row * D + d] = (bf16_t)(wsum > 0.f ? acc / wsum : 0.f);
+    out[row * D + d] = (bf16_t)(wsum > 0.f ? acc / wsum * gate_factor(gate, gate_stride, nq, row, d) : 0.f);
   }
 }
 
@@ -1223,7 +1241,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     const size_t row_index = tile_row0 + (size_t)rt * a.nq + kvh * g + rh;
     const float val = den > 0.f ? num / den : 0.f;
     if (a.num_splits == 1) {
-      a.out[row_index * D + d] = (bf16_t)val;
+      a.out[row_index * D + d] = (bf16_t)(val * gate_factor(a.gate, a.gate_stride, a.nq, row_index, d));
     } else {
       a.part_o[(row_index * a.num_splits + split) * D + d] = val;
       if (d == 0) a.part_lse[row_index * a.num_splits + split] = den > 0.f ? mm + log2f(den) : -INFINITY;
@@ -1269,6 +1287,8 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a mask of chunks, not both");
   QRT_CHECK((a.cap_in > 0.f) == (a.cap_out > 0.f), "attention: a score cap needs both of its factors");
+  QRT_CHECK(!a.gate || a.gate_stride >= (long)a.nq * D, "attention: the gate's rows are %ld elements apart, %d heads of %d need more",
+            a.gate_stride, a.nq, D);
   QRT_CHECK(a.items ? a.split_blocks > 0 && a.max_items >= a.num_tiles && a.max_items <= 65535
                     : a.split_blocks == 0,
             "attention (decode): pieces of %d blocks with a list of %d items for %d sequences", a.split_blocks,
@@ -1319,7 +1339,7 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
     const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
     if (merge_rows > 0)
       attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
-          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq);
+          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride);
     QRT_LAUNCH_CHECK("attention_merge");
   }
   return 0;
@@ -1337,6 +1357,8 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   QRT_CHECK(a.chunk >= 0 && !(a.chunk > 0 && a.window > 0), "attention: a window or a mask of chunks, not both");
   QRT_CHECK((a.cap_in > 0.f) == (a.cap_out > 0.f), "attention: a score cap needs both of its factors");
+  QRT_CHECK(!a.gate || a.gate_stride >= (long)a.nq * D, "attention: the gate's rows are %ld elements apart, %d heads of %d need more",
+            a.gate_stride, a.nq, D);
   if (a.num_tiles == 0) return 0;
   const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   QRT_CHECK((long long)a.num_tiles * a.nkv < (1ll << 31), "attention: %d tiles x %d key heads is too many blocks", a.num_tiles, a.nkv);
@@ -1376,7 +1398,7 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
     const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
     if (merge_rows > 0)
       attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
-          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq);
+          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq, a.gate, a.gate_stride);
     QRT_LAUNCH_CHECK("attention_merge");
   }
   return 0;

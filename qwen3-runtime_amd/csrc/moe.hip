@@ -18,6 +18,7 @@ __device__ __forceinline__ float lane_dot(const T* __restrict__ w, const float* 
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
   float acc = 0.f;
   if (wide) {
+#pragma unroll 4
     for (int c = lane * VEC; c < n; c += 64 * VEC) {
       const vec_t v = *(const vec_t*)(w + c);
 #pragma unroll
@@ -31,19 +32,33 @@ __device__ __forceinline__ float lane_dot(const T* __restrict__ w, const float* 
 
 // ------------------------------------------------------------------- router
 #define MAX_EXPERTS 1024
+// One block of 16 waves per token. A wave takes the experts wave, wave + 16, ...: its lanes read
+// the token's row and the expert's row straight from memory, several 16-byte pieces in flight
+// each, so that a router of 16 experts costs about two rounds of memory latency.
 template <typename T>
-__global__ __launch_bounds__(256) void route_top_kernel(const T* __restrict__ x, const float* __restrict__ router,
-                                                        const float* __restrict__ bias, int* __restrict__ index,
-                                                        float* __restrict__ weight, int hidden, int experts, int top) {
-  extern __shared__ float smem[];
-  float* xs = smem;               // [hidden]
-  float* logit = smem + hidden;   // [experts]
+__global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x, const float* __restrict__ router,
+                                                         const float* __restrict__ bias, int* __restrict__ index,
+                                                         float* __restrict__ weight, int hidden, int experts, int top) {
+  __shared__ float logit[MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int c = threadIdx.x; c < hidden; c += 256) xs[c] = to_f32<T>(x[(size_t)t * hidden + c]);
-  __syncthreads();
+  const T* xr = x + (size_t)t * hidden;
   const bool wide = hidden % 4 == 0;
-  for (int e = wave; e < experts; e += 4) {
-    const float z = wave_sum(lane_dot<float>(router + (size_t)e * hidden, xs, hidden, lane, wide));
+  for (int e = wave; e < experts; e += 16) {
+    const float* wr = router + (size_t)e * hidden;
+    float acc = 0.f;
+    if (wide) {
+      typedef T xvec_t __attribute__((ext_vector_type(4)));
+#pragma unroll 8
+      for (int c = lane * 4; c < hidden; c += 256) {
+        const f32x4_t wv = *(const f32x4_t*)(wr + c);
+        const xvec_t xv = *(const xvec_t*)(xr + c);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc = fmaf(to_f32<T>(xv[k]), wv[k], acc);
+      }
+    } else {
+      for (int c = lane; c < hidden; c += 64) acc = fmaf(to_f32<T>(xr[c]), wr[c], acc);
+    }
+    const float z = wave_sum(acc);
     if (lane == 0) logit[e] = z + (bias ? bias[e] : 0.f);
   }
   __syncthreads();
@@ -63,6 +78,7 @@ __global__ __launch_bounds__(256) void route_top_kernel(const T* __restrict__ x,
       const int oa = __shfl_xor(at, o, 64);
       if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
     }
+    at = min(at, experts - 1);  // logits that are not numbers compare false throughout: still an expert
     if (j == 0) first = best;
     const float p = expf(best - first);
     denom += p;
@@ -81,14 +97,12 @@ extern "C" int qrt_route_top(const void* x, int x_dtype, const float* router, co
   QRT_CHECK(num_tokens >= 0 && hidden > 0, "route_top: bad sizes T=%d H=%d", num_tokens, hidden);
   QRT_CHECK(experts >= 1 && experts <= MAX_EXPERTS && top >= 1 && top <= experts && top <= 64,
             "route_top: %d of %d experts (at most %d experts, 64 chosen)", top, experts, MAX_EXPERTS);
-  const size_t smem = (size_t)(hidden + experts) * sizeof(float);
-  QRT_CHECK(smem <= 64 * 1024, "route_top: rows of %d elements do not fit", hidden);
   if (num_tokens == 0) return 0;
-  dim3 grid(num_tokens), block(256);
+  dim3 grid(num_tokens), block(1024);
   if (x_dtype == QRT_F32)
-    route_top_kernel<float><<<grid, block, smem, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top);
+    route_top_kernel<float><<<grid, block, 0, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top);
   else if (x_dtype == QRT_BF16)
-    route_top_kernel<bf16_t><<<grid, block, smem, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top);
+    route_top_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top);
   else return qrt_fail("route_top: unknown dtype %d", x_dtype);
   QRT_LAUNCH_CHECK("route_top");
   return 0;
@@ -163,6 +177,212 @@ extern "C" int qrt_moe_pairs(const void* x, const void* gate_up, const void* dow
     moe_down_kernel<bf16_t><<<g2, 256, top * inter * 4, stream>>>((const bf16_t*)act, (const bf16_t*)down, index, weight, out, hidden, inter, top);
   }
   QRT_LAUNCH_CHECK("moe_pairs");
+  return 0;
+}
+
+// --------------------------------- experts, expert by expert (many tokens)
+// With many tokens each expert multiplies a matrix of its own tokens once: the pairs are put in
+// the order of their experts (group), the tokens' rows gathered in that order, the experts'
+// products run on their stretches of rows (the host's loop over the engine's own matrix
+// products, or one batched library product over stretches padded to equal length), and the
+// results weighted and summed per token (combine), pair by pair in the order of the router's
+// choice, without atomics on the output.
+//
+// group: order[i] = the pair at place i, place[p] = the place of pair p, offsets[e] = the first
+// place of expert e (offsets[E] = P). One block. Which of an expert's pairs gets which of its
+// places is left to the order in which the atomics arrive; no result depends on it, since
+// every row is computed by itself.
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ index, int* __restrict__ order,
+                                                         int* __restrict__ place, int* __restrict__ offsets,
+                                                         int pairs, int experts) {
+  __shared__ int count[MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e <= experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[index[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      const int n = count[e];
+      count[e] = at;
+      offsets[e] = at;
+      at += n;
+    }
+    offsets[experts] = at;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int at = atomicAdd(&count[index[p]], 1);
+    order[at] = p;
+    place[p] = at;
+  }
+}
+
+// The row of place `at` among the experts' rows: the place itself, or, where every expert has a
+// stretch of `padded` rows of its own (one batched product over all experts), the expert's
+// stretch plus the place within the expert.
+__device__ __forceinline__ size_t moe_row(int at, int expert, const int* __restrict__ offsets, int padded) {
+  return padded > 0 ? (size_t)expert * padded + (at - offsets[expert]) : (size_t)at;
+}
+
+template <typename T>
+__global__ void moe_gather_kernel(const T* __restrict__ x, const int* __restrict__ order, const int* __restrict__ index,
+                                  const int* __restrict__ offsets, int padded, T* __restrict__ xs, int hidden, int top) {
+  const int p = order[blockIdx.x];
+  const T* src = x + (size_t)(p / top) * hidden;
+  T* dst = xs + moe_row(blockIdx.x, index[p], offsets, padded) * hidden;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = src[c];
+}
+
+template <typename T>
+__global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ place, const int* __restrict__ index,
+                                   const int* __restrict__ offsets, int padded, const float* __restrict__ weight,
+                                   float* __restrict__ out, int hidden, int top) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) {
+      const size_t p = (size_t)t * top + j;
+      sum = fmaf(weight[p], to_f32<T>(y[moe_row(place[p], index[p], offsets, padded) * hidden + c]), sum);
+    }
+    out[(size_t)t * hidden + c] = sum;
+  }
+}
+
+extern "C" int qrt_moe_group(const int* index, int* order, int* place, int* offsets, int pairs, int experts,
+                             hipStream_t stream) {
+  QRT_CHECK(pairs > 0 && experts >= 1 && experts <= MAX_EXPERTS, "moe_group: bad sizes");
+  moe_group_kernel<<<1, 1024, 0, stream>>>(index, order, place, offsets, pairs, experts);
+  QRT_LAUNCH_CHECK("moe_group");
+  return 0;
+}
+
+extern "C" int qrt_moe_gather(const void* x, const int* order, const int* index, const int* offsets, int padded,
+                              void* xs, int dtype, int pairs, int hidden, int top, hipStream_t stream) {
+  QRT_CHECK(pairs > 0 && hidden > 0 && top > 0 && padded >= 0, "moe_gather: bad sizes");
+  if (dtype == QRT_F32) moe_gather_kernel<float><<<pairs, 256, 0, stream>>>((const float*)x, order, index, offsets, padded, (float*)xs, hidden, top);
+  else if (dtype == QRT_BF16) moe_gather_kernel<bf16_t><<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, index, offsets, padded, (bf16_t*)xs, hidden, top);
+  else return qrt_fail("moe_gather: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("moe_gather");
+  return 0;
+}
+
+extern "C" int qrt_moe_combine(const void* y, const int* place, const int* index, const int* offsets, int padded,
+                               const float* weight, float* out, int dtype, int num_tokens, int hidden, int top,
+                               hipStream_t stream) {
+  QRT_CHECK(num_tokens > 0 && hidden > 0 && top > 0 && padded >= 0, "moe_combine: bad sizes");
+  if (dtype == QRT_F32) moe_combine_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)y, place, index, offsets, padded, weight, out, hidden, top);
+  else if (dtype == QRT_BF16) moe_combine_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)y, place, index, offsets, padded, weight, out, hidden, top);
+  else return qrt_fail("moe_combine: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("moe_combine");
+  return 0;
+}
+
+// ------------------- experts, expert by expert, without the host (decoding in batches)
+// Once several tokens share an expert, the pair-by-pair form reads that expert's matrices once
+// per token. Here the pairs are grouped by expert on the device (moe_group above) and a block
+// owns a few rows of one expert's matrix: it brings them into LDS once and multiplies them
+// with every token of that expert, a token per wave at a time, the token's row read from
+// memory in 16-byte pieces. Blocks of experts that nobody chose leave at once. No count ever
+// reaches the host, so the form can be captured into a graph. GATED: the rows are R gate rows
+// and the R up rows that go with them, the input is the tokens' matrix and the output
+// silu(gate) * up by pair; otherwise R rows of the down matrix, the input by pair and the
+// output by place (moe_combine weighs and sums it). Every output element is one wave's sum in a
+// fixed order.
+template <typename T, int R, bool GATED>
+__global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __restrict__ in, const T* __restrict__ w,
+                                                                 const int* __restrict__ order,
+                                                                 const int* __restrict__ offsets, T* __restrict__ out,
+                                                                 int K, int N, int top) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int NR = GATED ? 2 * R : R;
+  typedef T vec_t __attribute__((ext_vector_type(VEC)));
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T* rows = (T*)smem_raw;  // [NR, K]
+  const int e = blockIdx.x, n0 = blockIdx.y * R;
+  const int first = offsets[e], count = offsets[e + 1] - first;
+  if (count == 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* we = w + (size_t)e * (GATED ? 2 : 1) * N * K;
+  for (int idx = threadIdx.x * VEC; idx < NR * K; idx += 256 * VEC) {
+    const int r = idx / K, c = idx - r * K;
+    const int n = min(n0 + (r % R), N - 1) + (GATED && r >= R ? N : 0);  // beyond the matrix: its last row, dropped below
+    *(vec_t*)(rows + idx) = *(const vec_t*)(we + (size_t)n * K + c);
+  }
+  __syncthreads();
+  for (int i = wave; i < count; i += 4) {
+    const int p = order[first + i];
+    const T* xr = in + (size_t)(GATED ? p / top : p) * K;
+    float acc[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) acc[r] = 0.f;
+#pragma unroll 2
+    for (int c = lane * VEC; c < K; c += 64 * VEC) {
+      const vec_t xv = *(const vec_t*)(xr + c);
+      float xf[VEC];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) xf[k] = to_f32<T>(xv[k]);
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const vec_t wv = *(const vec_t*)(rows + (size_t)r * K + c);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[r] = fmaf(xf[k], to_f32<T>(wv[k]), acc[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) acc[r] = wave_sum(acc[r]);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (n0 + r >= N) break;
+        if (GATED) out[(size_t)p * N + n0 + r] = from_f32<T>(acc[r] / (1.0f + expf(-acc[r])) * acc[R + r]);
+        else out[(size_t)(first + i) * N + n0 + r] = from_f32<T>(acc[r]);
+      }
+    }
+  }
+}
+
+template <typename T, int R, bool GATED>
+static void moe_rows_launch(const void* in, const void* w, const int* order, const int* offsets, void* out, int K, int N,
+                            int experts, int top, hipStream_t stream) {
+  dim3 grid(experts, (N + R - 1) / R);
+  const size_t smem = (size_t)(GATED ? 2 * R : R) * K * sizeof(T);
+  moe_rows_by_expert_kernel<T, R, GATED><<<grid, 256, smem, stream>>>((const T*)in, (const T*)w, order, offsets, (T*)out, K, N, top);
+}
+
+template <typename T, bool GATED>
+static int moe_rows_pick(const void* in, const void* w, const int* order, const int* offsets, void* out, int K, int N,
+                         int experts, int top, hipStream_t stream) {
+  // as many rows a block as 48 KB of LDS hold, eight at most
+  const size_t row_bytes = (size_t)(GATED ? 2 : 1) * K * sizeof(T);
+  const int fit = (int)(48 * 1024 / row_bytes);
+  if (fit >= 8) moe_rows_launch<T, 8, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
+  else if (fit >= 4) moe_rows_launch<T, 4, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
+  else if (fit >= 2) moe_rows_launch<T, 2, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
+  else if (fit >= 1) moe_rows_launch<T, 1, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
+  else return qrt_fail("moe: rows of %d elements do not fit the block's memory", K);
+  return 0;
+}
+
+// x [T, H] -> act [pairs, I] (by pair) -> y [pairs, H] (by place); order and offsets from qrt_moe_group
+extern "C" int qrt_moe_by_expert(const void* x, const void* gate_up, const void* down, const int* order,
+                                 const int* offsets, void* act, void* y, int dtype, int hidden, int inter, int experts,
+                                 int top, hipStream_t stream) {
+  QRT_CHECK(hidden > 0 && inter > 0 && experts >= 1 && experts <= MAX_EXPERTS && top > 0, "moe: bad sizes");
+  QRT_CHECK(dtype == QRT_F32 || dtype == QRT_BF16, "moe: unknown dtype %d", dtype);
+  const int vec = dtype == QRT_F32 ? 4 : 8;
+  QRT_CHECK(hidden % vec == 0 && inter % vec == 0, "moe: widths %d and %d are no multiples of %d", hidden, inter, vec);
+  QRT_CHECK((inter + 0) / 1 <= 65535 * 8 && hidden <= 65535 * 8, "moe: rows too many for one launch");
+  int rc;
+  if (dtype == QRT_F32) {
+    rc = moe_rows_pick<float, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, stream);
+    if (rc == 0) rc = moe_rows_pick<float, false>(act, down, order, offsets, y, inter, hidden, experts, top, stream);
+  } else {
+    rc = moe_rows_pick<bf16_t, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, stream);
+    if (rc == 0) rc = moe_rows_pick<bf16_t, false>(act, down, order, offsets, y, inter, hidden, experts, top, stream);
+  }
+  if (rc != 0) return rc;
+  QRT_LAUNCH_CHECK("moe_by_expert");
   return 0;
 }
 

@@ -80,6 +80,7 @@ class _AttnTileArgs(Structure):
         ("rope", c_void_p), ("slots", c_void_p), ("eps", c_float), ("split_blocks", c_int),
         ("max_items", c_int), ("items", c_void_p),
         ("chunk", c_int), ("cap_in", c_float), ("cap_out", c_float),
+        ("gate", c_void_p), ("gate_stride", c_long),
     ]
 
 
@@ -305,11 +306,74 @@ class HipOps:
         _need(down, "expert down", x.dtype, (n, h, inter))
         _need(index, "expert index", torch.int32, (t, top))
         _need(weight, "expert weight", torch.float32, (t, top))
-        act = torch.empty((t * top, inter), dtype=x.dtype, device=x.device)
         out = torch.empty((t, h), dtype=torch.float32, device=x.device)
+        if t == 0:
+            return out
+        pairs = t * top
+        if (pairs >= self.moe_grouped_min_pairs and pairs >= self.moe_grouped_pairs_per_expert * n
+                and not torch.cuda.is_current_stream_capturing()):
+            return self._moe_grouped(x, gate_up, down, index, weight, out)
+        act = torch.empty((t * top, inter), dtype=x.dtype, device=x.device)
+        vec = 16 // x.element_size()
+        if pairs >= self.moe_by_expert_pairs_per_expert * n and h % vec == 0 and inter % vec == 0:
+            # several tokens an expert: each expert's rows are read once, by blocks that own them
+            order = torch.empty(pairs, dtype=torch.int32, device=x.device)
+            place = torch.empty(pairs, dtype=torch.int32, device=x.device)
+            offsets = torch.empty(n + 1, dtype=torch.int32, device=x.device)
+            y = torch.empty((pairs, h), dtype=x.dtype, device=x.device)
+            self._check(self.lib, self.lib.qrt_moe_group(_ptr(index), _ptr(order), _ptr(place), _ptr(offsets),
+                                                         c_int(pairs), c_int(n), _stream()))
+            self._check(self.lib, self.lib.qrt_moe_by_expert(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(order), _ptr(offsets),
+                                                             _ptr(act), _ptr(y), _CODE[x.dtype], c_int(h), c_int(inter),
+                                                             c_int(n), c_int(top), _stream()))
+            self._check(self.lib, self.lib.qrt_moe_combine(_ptr(y), _ptr(place), _ptr(index), _ptr(offsets), c_int(0),
+                                                           _ptr(weight), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
+                                                           c_int(top), _stream()))
+            return out
         self._check(self.lib, self.lib.qrt_moe_pairs(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(index), _ptr(weight),
                                                      _ptr(act), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
                                                      c_int(inter), c_int(n), c_int(top), _stream()))
+        return out
+
+    # Steps of many tokens run the experts one by one, each on the rows of its own tokens, with
+    # the engine's matrix products (an expert's matrices are then read once, not once per pair):
+    # from this many pairs on, and from this many pairs per expert on. It reads the experts'
+    # row counts on the host, so a step that is being captured into a graph never takes it.
+    moe_grouped_min_pairs = 64
+    moe_grouped_pairs_per_expert = 4
+    # Steps that may not wait for the device (captured ones) and steps too small for that: from
+    # this many pairs per expert on, the experts' rows are read once per expert by a kernel that
+    # walks the expert's tokens; below it, once per pair (fewer launches, and pairs rarely meet).
+    moe_by_expert_pairs_per_expert = 1
+
+    def _moe_grouped(self, x, gate_up, down, index, weight, out):
+        t, h = x.shape
+        n, top = gate_up.shape[0], index.shape[1]
+        pairs = t * top
+        dev = x.device
+        order = torch.empty(pairs, dtype=torch.int32, device=dev)
+        place = torch.empty(pairs, dtype=torch.int32, device=dev)
+        offsets = torch.empty(n + 1, dtype=torch.int32, device=dev)
+        self._check(self.lib, self.lib.qrt_moe_group(_ptr(index), _ptr(order), _ptr(place), _ptr(offsets),
+                                                     c_int(pairs), c_int(n), _stream()))
+        bounds = offsets.cpu().tolist()  # the one wait of the step's host for the device
+        # The experts' rows lie one expert after the other (``padded`` = 0). The kernels also know a
+        # layout in which every expert has a stretch of equal length, made for one batched library
+        # product over all experts; that product is not used: the one run of it at the sizes of a
+        # real model ended in a fault of the device whose cause has not been found.
+        padded = 0
+        xs = torch.empty((pairs, h), dtype=x.dtype, device=dev)
+        self._check(self.lib, self.lib.qrt_moe_gather(_ptr(x), _ptr(order), _ptr(index), _ptr(offsets), c_int(padded),
+                                                      _ptr(xs), _CODE[x.dtype], c_int(pairs), c_int(h), c_int(top),
+                                                      _stream()))
+        y = torch.empty((pairs, h), dtype=x.dtype, device=dev)
+        for e in range(n):
+            a, b = bounds[e], bounds[e + 1]
+            if b > a:
+                y[a:b] = self.linear(self.gated_linear(xs[a:b], gate_up[e]), down[e])
+        self._check(self.lib, self.lib.qrt_moe_combine(_ptr(y), _ptr(place), _ptr(index), _ptr(offsets), c_int(padded),
+                                                       _ptr(weight), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
+                                                       c_int(top), _stream()))
         return out
 
     def sigmoid_gate(self, out, gate):
@@ -639,9 +703,7 @@ class HipOps:
                "rope": None if inv_freq is None else self.rope_table(ctx, inv_freq, angles_key)}
         out = torch.empty((t, nq * d), dtype=qkv.dtype, device=qkv.device)
         self._launch_attention(None, out, cache, ctx, nq, nkv, d, scale, window or 0, None, True, own,
-                               chunk=chunk or 0, softcap=softcap or 0.0)
-        if gate is not None:
-            self.sigmoid_gate(out, gate)
+                               chunk=chunk or 0, softcap=softcap or 0.0, gate=gate)
         return out
 
     def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window, chunk=None, softcap=None, value_dim=None,
@@ -665,9 +727,7 @@ class HipOps:
             raise OpsError(f"block table is {table.shape[1]} pages wide, the longest sequence needs {need_pages}")
         out = torch.empty((t, nq * dv), dtype=q.dtype, device=q.device)
         if dv == d and q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
-            self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0, chunk or 0, softcap or 0.0)
-            if gate is not None:
-                self.sigmoid_gate(out, gate)
+            self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0, chunk or 0, softcap or 0.0, gate)
         else:
             a = _AttnArgs()
             a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
@@ -803,7 +863,7 @@ class HipOps:
     # mixed steps: sequences with few rows leave the prompt kernel when their context is this long
     split_launch_min_kv = 1024
 
-    def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window, chunk=0, softcap=0.0):
+    def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window, chunk=0, softcap=0.0, gate=None):
         """Which kernel for which sequences. Steps of decoded tokens only: the decode kernel.
         Other steps: the prompt kernels; but sequences of at most 16 rows with a long context
         (decoded tokens beside a prompt portion) would each walk all their keys in one block
@@ -814,23 +874,24 @@ class HipOps:
         g = nq // nkv
         seqs = range(ctx.num_seqs)
         if ctx.max_q_len * g <= 16 and d <= 256:
-            return self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, True, chunk=chunk, softcap=softcap)
+            return self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, True, chunk=chunk, softcap=softcap, gate=gate)
         small = [s for s in seqs if ctx.q_lens_host[s] * g <= 16]
         if (d <= 256 and small and len(small) < ctx.num_seqs
                 and max(ctx.kv_lens_host[s] for s in small) >= self.split_launch_min_kv):
             small_set = set(small)
             big = [s for s in seqs if s not in small_set]
-            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, small, True, chunk=chunk, softcap=softcap)
-            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, big, False, chunk=chunk, softcap=softcap)
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, small, True, chunk=chunk, softcap=softcap, gate=gate)
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, big, False, chunk=chunk, softcap=softcap, gate=gate)
             return
-        self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False, chunk=chunk, softcap=softcap)
+        self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False, chunk=chunk, softcap=softcap, gate=gate)
 
     def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode, own=None,
-                          chunk=0, softcap=0.0):
+                          chunk=0, softcap=0.0, gate=None):
         """One launch over the sequences in ``subset`` (None: all of the step's). ``own``: the
         decode kernel takes the tokens' queries, own keys and own values from the q/k/v product
         (``decode_attention``); ``q`` is then None. ``chunk``: a mask of chunks in place of a
-        window; ``softcap``: the cap on the scaled scores."""
+        window; ``softcap``: the cap on the scaled scores; ``gate`` [T, nq * d] (columns of a wider
+        matrix will do): its sigmoid multiplies the output where the kernels write it."""
         lib = attention_library(d)
         # how far back a query can see at most: what the choices below (key splits, pieces) go by
         reach = window or chunk
@@ -877,6 +938,10 @@ class HipOps:
         a.chunk = chunk
         if softcap:
             a.cap_in, a.cap_out = scale / softcap, softcap / scale
+        if gate is not None:
+            if gate.dtype != torch.bfloat16 or tuple(gate.shape) != (ctx.num_tokens, nq * d) or gate.stride(1) != 1:
+                raise OpsError(f"gate {tuple(gate.shape)} {gate.dtype} does not fit {ctx.num_tokens} tokens of {nq} heads of {d}")
+            a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
         piece = None
         if decode and n_tiles <= 1024:
             piece = ctx.scratch.get("attn_piece")  # keys per piece, a multiple of 32: asked for outright

@@ -115,8 +115,12 @@ def test_router_takes_the_best_and_weighs_them_among_themselves(backend, experts
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("experts,top,width,inner,tokens", [(8, 2, 256, 64, 11), (5, 3, 96, 40, 4), (3, 1, 128, 48, 70),
-                                                            (4, 4, 64, 32, 1), (6, 2, 128, 96, 300)])
+                                                            (4, 4, 64, 32, 1), (6, 2, 128, 96, 300), (16, 2, 128, 64, 3),
+                                                            (7, 2, 100, 36, 9)])
 def test_experts_weighted_sum(backend, experts, top, width, inner, tokens):
+    """The three forms the device has: pair by pair (fewer pairs than experts, or widths without
+    16-byte pieces), expert by expert on the device (several pairs an expert), and expert by
+    expert through the engine's matrix products (many tokens)."""
     device, dtype = backend
     ops = make_ops(device)
     x = rnd(tokens, width, seed=1).to(DT[dtype])
