@@ -304,10 +304,17 @@ __global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __rest
   if (count == 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* we = w + (size_t)e * (GATED ? 2 : 1) * N * K;
-  for (int idx = threadIdx.x * VEC; idx < NR * K; idx += 256 * VEC) {
-    const int r = idx / K, c = idx - r * K;
-    const int n = min(n0 + (r % R), N - 1) + (GATED && r >= R ? N : 0);  // beyond the matrix: its last row, dropped below
-    *(vec_t*)(rows + idx) = *(const vec_t*)(we + (size_t)n * K + c);
+  // all NR rows' pieces of a column range are asked for before the first is stored: NR loads in
+  // flight a thread, and a row of 2,560 elements is through in two such rounds
+  for (int c = threadIdx.x * VEC; c < K; c += 256 * VEC) {
+    vec_t piece[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      const int n = min(n0 + (r % R), N - 1) + (GATED && r >= R ? N : 0);  // beyond the matrix: its last row, dropped below
+      piece[r] = *(const vec_t*)(we + (size_t)n * K + c);
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) *(vec_t*)(rows + (size_t)r * K + c) = piece[r];
   }
   __syncthreads();
   for (int i = wave; i < count; i += 4) {

@@ -367,9 +367,26 @@ class HipOps:
                                                       _ptr(xs), _CODE[x.dtype], c_int(pairs), c_int(h), c_int(top),
                                                       _stream()))
         y = torch.empty((pairs, h), dtype=x.dtype, device=dev)
-        for e in range(n):
-            a, b = bounds[e], bounds[e + 1]
-            if b > a:
+        busy = [(e, bounds[e], bounds[e + 1]) for e in range(n) if bounds[e + 1] > bounds[e]]
+        if x.dtype == torch.bfloat16:
+            # what bounds this form is the host's time per launch, so an expert costs two of them:
+            # its products go straight into its rows of one buffer each (the library's for more
+            # rows than the engine's own kernels take), and one activation kernel serves all experts
+            inter = gate_up.shape[1] // 2
+            both = torch.empty((pairs, 2 * inter), dtype=x.dtype, device=dev)
+            for e, a, b in busy:
+                if b - a > self.own_max_rows:
+                    torch.mm(xs[a:b], gate_up[e].t(), out=both[a:b])
+                else:
+                    both[a:b] = self.linear(xs[a:b], gate_up[e])
+            act = self.swiglu(both)
+            for e, a, b in busy:
+                if b - a > self.own_max_rows:
+                    torch.mm(act[a:b], down[e].t(), out=y[a:b])
+                else:
+                    y[a:b] = self.linear(act[a:b], down[e])
+        else:
+            for e, a, b in busy:
                 y[a:b] = self.linear(self.gated_linear(xs[a:b], gate_up[e]), down[e])
         self._check(self.lib, self.lib.qrt_moe_combine(_ptr(y), _ptr(place), _ptr(index), _ptr(offsets), c_int(padded),
                                                        _ptr(weight), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),

@@ -404,6 +404,57 @@ def test_greedy_generation_through_the_entry_point(folder, name, dtype, graphs):
         assert int((below >= bound).sum()) <= allowed, (float(below.max()), int(below.argmax()))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_command_line_and_trace_replay(folder, tmp_path, dtype):
+    """As a user runs them: ``python -m qwen3_runtime_amd.cli --model DIR`` generates greedily, and
+    ``bin/trace_run`` replays a mixed schedule from standard input and writes the logits it is
+    asked for, with a pool that only holds what is live."""
+    import ast
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parents[1]
+    raw, page = config_d()
+    cfg, w = P.read_model(folder("d"))
+    prompt = [5, 17, 3, 140, 9, 77, 2]
+    proc = subprocess.run([sys.executable, "-m", "qwen3_runtime_amd.cli", "--model", str(folder("d")), "--dtype", dtype,
+                           "--prompt-tokens", *map(str, prompt), "--max-tokens", "8"],
+                          capture_output=True, text=True, timeout=600, cwd=str(root))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = dict(line.split(" ", 1) for line in proc.stdout.splitlines() if " " in line)
+    tokens = ast.literal_eval(lines["runtime"])
+    assert len(tokens) == 8
+    logits = P.forward(cfg, w, prompt + tokens)[len(prompt) - 1: -1]
+    below = logits.max(-1).values - logits[range(8), tokens]
+    assert float(below.max()) < (1e-3 if dtype == "float32" else 0.1 * float(logits.std()))
+
+    reqs = traces.make_requests(raw["vocab"], [70, 9, 41, 100, 35], seed=6)
+    steps = traces.mixed(reqs, seed=1)
+    out = tmp_path / "logits"
+    proc = subprocess.run([str(root / "bin" / "trace_run"), "--model", str(folder("d")), "--dtype", dtype, "--out", str(out),
+                           "--max-tokens", str(traces.peak_tokens(steps))],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True,
+                          timeout=600, cwd=str(root))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert [line for line in proc.stdout.splitlines() if line.startswith("done ")] == [f"done {s['step']}" for s in steps]
+    got, pos = {}, {r: 0 for r in reqs}
+    for s in steps:
+        wanted = sum(len(e["want"]) for e in s["entries"])
+        rows = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(wanted, raw["vocab"]) if wanted else None
+        i = 0
+        for e in s["entries"]:
+            for k in e["want"]:
+                got[(e["id"], pos[e["id"]] + k)] = torch.from_numpy(rows[i].copy())
+                i += 1
+            pos[e["id"]] += len(e["tokens"])
+    check(got, plain_logits(folder("d"), reqs), dtype, flips=FLIPS["d"])
+
+
 # ------------------------------------------------------------------ host side only
 def test_config_reader_and_plan():
     from qwen3_runtime_amd.config.deginex import DeginexConfig
