@@ -47,11 +47,11 @@ class AttentionSizes:
 
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any], where: str) -> "AttentionSizes":
-        for key in ("heads", "kv_heads", "dim", "scale"):
+        for key in ("heads", "dim", "scale"):
             if key not in raw:
                 raise ConfigError(f"{where}: the mixer lacks {key!r}")
         heads = _positive(where, "heads", raw["heads"])
-        kv_heads = _positive(where, "kv_heads", raw["kv_heads"])
+        kv_heads = _positive(where, "kv_heads", raw.get("kv_heads", heads))  # absent: a key head per query head
         if heads % kv_heads:
             raise ConfigError(f"{where}: {heads} query heads do not divide into {kv_heads} key/value heads")
         dim = _positive(where, "dim", raw["dim"])

@@ -51,13 +51,17 @@ def _feed_forward(cfg: DeginexConfig, sizes: FeedForwardSizes | None, p: str) ->
 
 
 def plan_deginex(cfg: DeginexConfig) -> ModelPlan:
-    layers = []
+    layers, unread = [], []
     for i, layer in enumerate(cfg.layers):
         p = f"l{i}"
         ff = _feed_forward(cfg, layer.feed_forward, p)
         norms = {"input": _norm(cfg, f"{p}.norm1")}
         if ff is not None:
             norms["post_mixer"] = _norm(cfg, f"{p}.norm2")
+        else:
+            # a layer without feed-forward has no second sub-layer: a file may still carry the norm
+            # and the stream coefficients that would have gone with it; they are not read
+            unread += [f"{p}.norm2", f"{p}.norm2.b"] + [f"{p}.hc2.{kind}" for kind in ("in", "out", "mix")]
         if cfg.streams is None:
             block = PartSpec("pre_norm")
         else:
@@ -77,6 +81,7 @@ def plan_deginex(cfg: DeginexConfig) -> ModelPlan:
         layers=layers, caches=caches, order=order,
         final_norm=_norm(cfg, "final.norm", cfg.streams or 1),
         head=PartSpec("linear_head", sizes, {"weight": "embed"}),
+        ignorable=tuple(unread),
         eos_token_id=cfg.eos_token_id,
     )
 

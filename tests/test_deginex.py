@@ -173,7 +173,8 @@ def attention_ctx(ops, device, dtype, q_len, kv_len):
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("heads,kv_heads,d,dv,chunk,cap,page", [(4, 2, 64, 64, 96, 20.0, 16), (6, 3, 16, 48, 24, 8.0, 8),
                                                                 (3, 3, 32, 32, None, None, 16), (8, 1, 32, 32, 40, 30.0, 8),
-                                                                (4, 4, 128, 128, 50, None, 16), (2, 1, 64, 64, 7, 5.0, 8)])
+                                                                (4, 4, 128, 128, 50, None, 16), (2, 1, 64, 64, 7, 5.0, 8),
+                                                                (2, 2, 64, 64, 1, 5.0, 8), (17, 1, 32, 32, 300, 12.0, 16)])
 @pytest.mark.parametrize("q_len,kv_len", [(1, 1), (1, 97), (1, 250), (5, 5), (33, 130), (200, 200), (2, 98), (70, 333)])
 def test_attention_chunks_cap_gate(backend, heads, kv_heads, d, dv, chunk, cap, page, q_len, kv_len):
     """Random queries over a paged sequence, against the plain scores, mask, cap, softmax and gate;
@@ -271,11 +272,27 @@ def config_d():
                        {"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": 96}}]}, 8
 
 
-CONFIGS = {"a": config_a, "b": config_b, "c": config_c, "d": config_d}
+def config_e():
+    """Sizes that fit no kernel's favourite shapes: a width and inner widths that are no multiples
+    of 8, keys of 24 and values of 40 elements, 17 query heads to a key head, five streams, a chunk
+    of 13 positions, every expert taken, an odd vocabulary."""
+    return {"architecture": "Deginex", "vocab": 77, "width": 100, "norm": {"eps": 1e-5}, "streams": 5,
+            "loop": {"start": 0, "stop": 1, "times": 2},
+            "layers": [{"type": "attention",
+                        "mixer": {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 40, "scale": 0.3, "softcap": 9.0,
+                                  "mask": {"size": 13}},
+                        "mlp": {"kind": "moe", "expert": {"ff": 20}, "router": {"experts": 3, "top": 3}}},
+                       {"type": "attention",
+                        "mixer": {"heads": 34, "kv_heads": 2, "dim": 16, "vdim": 16, "scale": 0.2, "mask": {"size": 64}},
+                        "mlp": {"kind": "dense", "ff": 52}}]}, 8
+
+
+CONFIGS = {"a": config_a, "b": config_b, "c": config_c, "d": config_d, "e": config_e}
 # share of positions at which a router may choose differently in bfloat16 (three routed runs a
 # token in "a", one in "b" and "c", none in "d")
-FLIPS = {"a": 0.09, "b": 0.03, "c": 0.03, "d": 0.0}
-LENGTHS = {"a": [1, 7, 45, 130], "b": [3, 17, 50, 64, 101], "c": [2, 16, 17, 49], "d": [5, 33, 34, 70]}
+FLIPS = {"a": 0.09, "b": 0.03, "c": 0.03, "d": 0.0, "e": 0.0}
+LENGTHS = {"a": [1, 7, 45, 130], "b": [3, 17, 50, 64, 101], "c": [2, 16, 17, 49], "d": [5, 33, 34, 70],
+           "e": [1, 13, 14, 66, 90]}
 _folders: dict = {}
 
 
@@ -481,6 +498,26 @@ def test_config_reader_and_plan():
     bad = {**raw, "layers": [{"type": "recurrence", "mixer": {}, "mlp": None}]}
     with pytest.raises(ConfigError, match="mixer type"):
         DeginexConfig.from_dict(bad)
+
+
+def test_a_file_may_carry_what_a_layer_without_feed_forward_does_not_read(folder, tmp_path):
+    import shutil
+
+    from safetensors.torch import load_file, save_file
+
+    from qwen3_runtime_amd.weights.loader import WeightError
+
+    src = folder("d")   # its first layer is a mixer alone
+    tensors = load_file(str(src / "model.safetensors"))
+    tensors["l0.norm2"] = torch.ones(128, dtype=torch.bfloat16)
+    tensors["l0.norm2.b"] = torch.zeros(128, dtype=torch.bfloat16)
+    shutil.copy(src / "config.json", tmp_path / "config.json")
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    load(tmp_path, 8, 8, ("cpu", "float32"))
+    tensors["l1.surplus"] = torch.ones(3, dtype=torch.bfloat16)
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightError, match="l1.surplus"):
+        load(tmp_path, 8, 8, ("cpu", "float32"))
 
 
 def test_pages_of_finished_chunks_go_back():
