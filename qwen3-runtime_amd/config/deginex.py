@@ -47,7 +47,7 @@ class AttentionSizes:
 
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any], where: str) -> "AttentionSizes":
-        for key in ("heads", "dim", "scale"):
+        for key in ("heads", "dim"):
             if key not in raw:
                 raise ConfigError(f"{where}: the mixer lacks {key!r}")
         heads = _positive(where, "heads", raw["heads"])
@@ -56,7 +56,7 @@ class AttentionSizes:
             raise ConfigError(f"{where}: {heads} query heads do not divide into {kv_heads} key/value heads")
         dim = _positive(where, "dim", raw["dim"])
         vdim = _positive(where, "vdim", raw.get("vdim", dim))
-        scale = float(raw["scale"])
+        scale = float(raw.get("scale", dim ** -0.5))  # absent: the usual 1 / sqrt(dim)
         if not scale > 0.0:
             raise ConfigError(f"{where}: scale must be positive, got {scale!r}")
         softcap = raw.get("softcap")
