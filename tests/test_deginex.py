@@ -139,6 +139,18 @@ def test_experts_weighted_sum(backend, experts, top, width, inner, tokens):
     torch.testing.assert_close(got.double().cpu(), want, **tol(dtype))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sigmoid_gate_on_columns_of_a_wider_matrix(dtype):
+    """The gate as a step of its own (the attention kernels apply it themselves; an attention that
+    cannot asks for this one)."""
+    ops = make_ops("cuda:0")
+    out, wide = rnd(7, 96, seed=1).to(DT[dtype]), rnd(7, 96 + 40, seed=2).to(DT[dtype])
+    want = out.double() * torch.sigmoid(wide[:, 40:].double())
+    got = ops.sigmoid_gate(out.to("cuda:0"), wide.to("cuda:0")[:, 40:])
+    torch.testing.assert_close(got.double().cpu(), want, **(tol(dtype) if dtype == "float32" else dict(atol=2e-2, rtol=2e-2)))
+
+
 def paged(keys, values, page_size, device, dtype, seed=0, spare=3):
     """Put one sequence's keys [n, heads, d] and values [n, heads, dv] into pages in a random
     order among spare ones that are poisoned; returns (view, table)."""
