@@ -334,6 +334,19 @@ class CacheManager:
     def group_of_cache(self, cache_id: int) -> int | None:
         return self._group_of_cache.get(cache_id)
 
+    def step_views(self, order, group_views: Sequence[GroupView]) -> list:
+        """What each step of a plan's ``order`` sees: None, a ``CacheView``, or a tuple of them for
+        a step that names several caches."""
+        views = []
+        for st in order:
+            if st.cache is None:
+                views.append(None)
+            elif isinstance(st.cache, (tuple, list)):
+                views.append(tuple(self.view(c, group_views, st.writes_cache) for c in st.cache))
+            else:
+                views.append(self.view(st.cache, group_views, st.writes_cache))
+        return views
+
     def view(self, cache_id: int, group_views: Sequence[GroupView], writes: bool = True) -> CacheView:
         spec = self.specs[cache_id]
         if spec.kind == "state":

@@ -1,0 +1,114 @@
+// Small float32 steps between sub-layers that are neither a product nor a plain norm:
+// the mean of several outputs each RMS-normed first (mixers side by side), the residual
+// stream joined with the embedding for a product that re-enters it (a looped span's entry),
+// a sum of two sub-layer outputs (routed and shared experts), and gated activations other than
+// SwiGLU. Inputs that are sub-layer outputs may be one matrix [T, H] (float32 or bfloat16) or
+// float32 planes [P, T, H] whose sum they are.
+#include "common.h"
+#include <math.h>
+
+struct Planes {
+  const void* p; int code; int planes; long plane_stride;
+};
+
+__device__ __forceinline__ float planes_at(const Planes& y, size_t i) {
+  if (y.code == QRT_BF16) return (float)((const bf16_t*)y.p)[i];
+  float v = 0.f;
+  for (int k = 0; k < y.planes; ++k) v += ((const float*)y.p)[(size_t)k * y.plane_stride + i];
+  return v;
+}
+
+// out[t] = (1/2) (a[t] / rms(a[t]) * wa + b[t] / rms(b[t]) * wb), rms with eps inside the root
+__global__ __launch_bounds__(256) void norm_mean_kernel(Planes ya, Planes yb, const float* __restrict__ wa,
+                                                        const float* __restrict__ wb, float* __restrict__ out,
+                                                        int hidden, float eps) {
+  __shared__ float red[32];
+  const size_t row = (size_t)blockIdx.x * hidden;
+  float sa = 0.f, sb = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    const float va = planes_at(ya, row + i), vb = planes_at(yb, row + i);
+    sa += va * va;
+    sb += vb * vb;
+  }
+  const float ia = 1.0f / sqrtf(block_sum(sa, red) / (float)hidden + eps);
+  const float ib = 1.0f / sqrtf(block_sum(sb, red) / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += 256)
+    out[row + i] = 0.5f * (planes_at(ya, row + i) * ia * wa[i] + planes_at(yb, row + i) * ib * wb[i]);
+}
+
+extern "C" int qrt_norm_mean(const void* a, int a_code, int a_planes, const void* b, int b_code, int b_planes,
+                             const float* wa, const float* wb, float* out, int num_tokens, int hidden, float eps,
+                             hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && hidden > 0 && a_planes >= 1 && b_planes >= 1, "norm_mean: bad sizes");
+  QRT_CHECK((a_code == QRT_F32 || (a_code == QRT_BF16 && a_planes == 1)) && (b_code == QRT_F32 || (b_code == QRT_BF16 && b_planes == 1)),
+            "norm_mean: planes are float32");
+  if (num_tokens == 0) return 0;
+  const long stride = (long)num_tokens * hidden;
+  norm_mean_kernel<<<dim3(num_tokens), 256, 0, stream>>>(Planes{a, a_code, a_planes, stride}, Planes{b, b_code, b_planes, stride},
+                                                         wa, wb, out, hidden, eps);
+  QRT_LAUNCH_CHECK("norm_mean");
+  return 0;
+}
+
+// out[t] = [ residual[t] + scale * delta[t] | origin[t] ]   (2H wide, in the products' type)
+template <typename TO>
+__global__ void add_concat_kernel(const float* __restrict__ residual, Planes delta, float scale,
+                                  const float* __restrict__ origin, TO* __restrict__ out, int hidden) {
+  const size_t row = (size_t)blockIdx.x * hidden;
+  TO* o = out + 2 * row;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = residual[row + i];
+    if (delta.p) v = fmaf(scale, planes_at(delta, row + i), v);
+    o[i] = from_f32<TO>(v);
+    o[hidden + i] = from_f32<TO>(origin[row + i]);
+  }
+}
+
+extern "C" int qrt_add_concat(const float* residual, const void* delta, int d_code, int d_planes, float scale,
+                              const float* origin, void* out, int out_dtype, int num_tokens, int hidden,
+                              hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && hidden > 0 && d_planes >= 1, "add_concat: bad sizes");
+  QRT_CHECK(!delta || d_code == QRT_F32 || (d_code == QRT_BF16 && d_planes == 1), "add_concat: planes are float32");
+  if (num_tokens == 0) return 0;
+  const Planes d{delta, d_code, d_planes, (long)num_tokens * hidden};
+  if (out_dtype == QRT_F32) add_concat_kernel<float><<<dim3(num_tokens), 256, 0, stream>>>(residual, d, scale, origin, (float*)out, hidden);
+  else if (out_dtype == QRT_BF16) add_concat_kernel<bf16_t><<<dim3(num_tokens), 256, 0, stream>>>(residual, d, scale, origin, (bf16_t*)out, hidden);
+  else return qrt_fail("add_concat: unknown dtype %d", out_dtype);
+  QRT_LAUNCH_CHECK("add_concat");
+  return 0;
+}
+
+// acc[t] += y[t]
+__global__ void accumulate_kernel(float* __restrict__ acc, Planes y, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) acc[i] += planes_at(y, (size_t)i);
+}
+
+extern "C" int qrt_accumulate(float* acc, const void* y, int y_code, int y_planes, long n, hipStream_t stream) {
+  QRT_CHECK(n >= 0 && y_planes >= 1, "accumulate: bad sizes");
+  QRT_CHECK(y_code == QRT_F32 || (y_code == QRT_BF16 && y_planes == 1), "accumulate: planes are float32");
+  if (n == 0) return 0;
+  accumulate_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, stream>>>(acc, Planes{y, y_code, y_planes, n}, n);
+  QRT_LAUNCH_CHECK("accumulate");
+  return 0;
+}
+
+// out[t, i] = act(gu[t, i], gu[t, I + i]) for the gated activations of common.h
+template <typename T>
+__global__ void gated_act_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int kind, float limit) {
+  const T* row = gu + (size_t)blockIdx.x * 2 * inter;
+  for (int i = threadIdx.x; i < inter; i += blockDim.x)
+    out[(size_t)blockIdx.x * inter + i] = from_f32<T>(gated_act(to_f32<T>(row[i]), to_f32<T>(row[inter + i]), kind, limit));
+}
+
+extern "C" int qrt_gated_act(const void* gu, void* out, int dtype, int num_tokens, int inter, int kind, float limit,
+                             hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && inter > 0, "gated_act: bad sizes");
+  QRT_CHECK(kind == QRT_ACT_SWIGLU || kind == QRT_ACT_CLAMPED, "gated_act: unknown activation %d", kind);
+  if (num_tokens == 0) return 0;
+  if (dtype == QRT_F32) gated_act_kernel<float><<<dim3(num_tokens), 256, 0, stream>>>((const float*)gu, (float*)out, inter, kind, limit);
+  else if (dtype == QRT_BF16) gated_act_kernel<bf16_t><<<dim3(num_tokens), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, kind, limit);
+  else return qrt_fail("gated_act: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("gated_act");
+  return 0;
+}

@@ -69,6 +69,19 @@ __device__ __forceinline__ void sincos_angle(float angle, float* sn, float* cs) 
   sincosf(reduced, sn, cs);
 }
 
+// Gated activations of feed-forwards, float32. SWIGLU: silu(g) u. CLAMPED: g and u are held to
+// `limit` first (g from above only, u from both sides), then g sigmoid(1.702 g) (u + 1).
+#define QRT_ACT_SWIGLU 0
+#define QRT_ACT_CLAMPED 1
+__device__ __forceinline__ float gated_act(float g, float u, int kind, float limit) {
+  if (kind == QRT_ACT_CLAMPED) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+  }
+  return g / (1.0f + expf(-g)) * u;
+}
+
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);

@@ -58,7 +58,7 @@ extern "C" int qrt_rope_table(const int* positions, const float* inv_freq, float
 
 // ------------------------------------------------------- add + RMSNorm
 // r = rows ? rows[b] : b
-// x = residual[r] (+ delta[r]);  without `rows` the sum is written back.
+// x = residual[r] (+ dscale * delta[r]);  without `rows` the sum is written back.
 // out[b] = x * rsqrt(mean(x^2) + eps) * weight
 // One block of 256 threads per row. Each thread keeps its elements of the row in registers
 // (rows up to 256 * VEC * KEEP wide; wider rows are read a second time), all loads of a row are
@@ -72,7 +72,8 @@ template <typename TD, typename TO, int VEC, int KEEP, int PL>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                                           const float* __restrict__ weight,
                                                           const int* __restrict__ rows, TO* __restrict__ out,
-                                                          int hidden, float eps, int planes, size_t plane_stride) {
+                                                          int hidden, float eps, int planes, size_t plane_stride,
+                                                          float dscale) {
   typedef float fvec_t __attribute__((ext_vector_type(VEC)));
   typedef TD dvec_t __attribute__((ext_vector_type(VEC)));
   typedef TO ovec_t __attribute__((ext_vector_type(VEC)));
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
 #pragma unroll
       for (int j = 0; j < KEEP; ++j)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) x[j][e] += to_f32<TD>(d[p][j][e]);
+        for (int e = 0; e < VEC; ++e) x[j][e] = fmaf(dscale, to_f32<TD>(d[p][j][e]), x[j][e]);
   } else {
 #pragma unroll
     for (int j = 0; j < KEEP; ++j) {
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
           const int ic = min(i0 + j * STRIDE, hidden - VEC);
           const dvec_t d = *(const dvec_t*)(del + p * plane_stride + ic);
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) x[j][e] += to_f32<TD>(d[e]);
+          for (int e = 0; e < VEC; ++e) x[j][e] = fmaf(dscale, to_f32<TD>(d[e]), x[j][e]);
         }
       }
     }
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
       for (int p = 0; p < planes; ++p) {
         const dvec_t d = *(const dvec_t*)(del + p * plane_stride + i);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[e] += to_f32<TD>(d[e]);
+        for (int e = 0; e < VEC; ++e) v[e] = fmaf(dscale, to_f32<TD>(d[e]), v[e]);
       }
       if (write_back) *(fvec_t*)(res + i) = v;
     }
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
       for (int p = 0; p < planes; ++p) {
         const dvec_t d = *(const dvec_t*)(del + p * plane_stride + i);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[e] += to_f32<TD>(d[e]);
+        for (int e = 0; e < VEC; ++e) v[e] = fmaf(dscale, to_f32<TD>(d[e]), v[e]);
       }
     }
     const fvec_t wv = *(const fvec_t*)(weight + i);
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
 
 extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const float* weight,
                                const int* rows, void* out, int out_dtype, int num_out_rows, int hidden,
-                               float eps, int planes, long plane_stride, hipStream_t stream) {
+                               float eps, int planes, long plane_stride, float dscale, hipStream_t stream) {
   QRT_CHECK(hidden > 0 && num_out_rows >= 0, "add_rmsnorm: bad sizes rows=%d H=%d", num_out_rows, hidden);
   QRT_CHECK(planes >= 1 && planes <= 64 && plane_stride >= 0, "add_rmsnorm: bad delta planes %d", planes);
   if (num_out_rows == 0) return 0;
@@ -188,7 +189,7 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
 #define GO(TD, TO, VEC, KEEP, PL)                                                                               \
   add_rmsnorm_kernel<TD, TO, VEC, KEEP, PL><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight,     \
                                                                         rows, (TO*)out, hidden, eps, planes,    \
-                                                                        (size_t)plane_stride)
+                                                                        (size_t)plane_stride, dscale)
 #define LAUNCH(TD, TO)                                                                                          \
   do {                                                                                                          \
     if (!vec4) GO(TD, TO, 1, 8, -1);                                                                            \

@@ -38,8 +38,10 @@ __device__ __forceinline__ float lane_dot(const T* __restrict__ w, const float* 
 template <typename T>
 __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x, const float* __restrict__ router,
                                                          const float* __restrict__ bias, int* __restrict__ index,
-                                                         float* __restrict__ weight, int hidden, int experts, int top) {
+                                                         float* __restrict__ weight, int hidden, int experts, int top,
+                                                         int sigmoid_scores, int groups, int keep) {
   __shared__ float logit[MAX_EXPERTS];
+  __shared__ float score[MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* xr = x + (size_t)t * hidden;
   const bool wide = hidden % 4 == 0;
@@ -63,6 +65,41 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
   }
   __syncthreads();
   if (wave != 0) return;
+  if (sigmoid_scores) {
+    // scores sigmoid(z) take the logits' place: the choice goes by them, and they are the weights
+    for (int e = lane; e < experts; e += 64) score[e] = logit[e] = 1.0f / (1.0f + expf(-logit[e]));
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (groups > 1 && keep < groups) {
+    // experts form `groups` equal groups of neighbours; a group's score is the sum of its two
+    // largest entries (of its one, if it has one); only the `keep` best groups stay in the choice
+    const int per = experts / groups;
+    float mine = -INFINITY;  // lane g holds group g's score (groups <= 64)
+    if (lane < groups) {
+      float a = -INFINITY, b = -INFINITY;
+      for (int e = lane * per; e < (lane + 1) * per; ++e) {
+        const float z = logit[e];
+        if (z > a) { b = a; a = z; } else if (z > b) b = z;
+      }
+      mine = per > 1 ? a + b : a;
+    }
+    bool kept = false;
+    for (int j = 0; j < keep; ++j) {
+      float best = kept ? -INFINITY : mine;
+      int at = (kept || lane >= groups) ? 0x7fffffff : lane;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const int oa = __shfl_xor(at, o, 64);
+        if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+      }
+      if (lane == at) kept = true;
+    }
+    const unsigned long long mask = __ballot(kept);
+    for (int e = lane; e < experts; e += 64)
+      if (!((mask >> (e / per)) & 1ull)) logit[e] = -INFINITY;
+    __builtin_amdgcn_wave_barrier();
+  }
   // `top` rounds of "largest that is left", ties to the lower index
   float chosen = 0.f, first = 0.f, denom = 0.f;
   for (int j = 0; j < top; ++j) {
@@ -80,7 +117,7 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
     }
     at = min(at, experts - 1);  // logits that are not numbers compare false throughout: still an expert
     if (j == 0) first = best;
-    const float p = expf(best - first);
+    const float p = sigmoid_scores ? score[at] : expf(best - first);
     denom += p;
     if (lane == j) chosen = p;
     if (lane == 0) {
@@ -89,20 +126,24 @@ __global__ __launch_bounds__(1024) void route_top_kernel(const T* __restrict__ x
     }
     __builtin_amdgcn_wave_barrier();
   }
-  if (lane < top) weight[(size_t)t * top + lane] = chosen / denom;
+  if (lane < top) weight[(size_t)t * top + lane] = sigmoid_scores ? chosen : chosen / denom;
 }
 
 extern "C" int qrt_route_top(const void* x, int x_dtype, const float* router, const float* bias, int* index,
-                             float* weight, int num_tokens, int hidden, int experts, int top, hipStream_t stream) {
+                             float* weight, int num_tokens, int hidden, int experts, int top, int sigmoid_scores,
+                             int groups, int keep, hipStream_t stream) {
+  QRT_CHECK(groups >= 1 && groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups &&
+            (long)keep * (experts / groups) >= top,
+            "route_top: %d groups of which %d stay do not fit %d experts of which %d are chosen", groups, keep, experts, top);
   QRT_CHECK(num_tokens >= 0 && hidden > 0, "route_top: bad sizes T=%d H=%d", num_tokens, hidden);
   QRT_CHECK(experts >= 1 && experts <= MAX_EXPERTS && top >= 1 && top <= experts && top <= 64,
             "route_top: %d of %d experts (at most %d experts, 64 chosen)", top, experts, MAX_EXPERTS);
   if (num_tokens == 0) return 0;
   dim3 grid(num_tokens), block(1024);
   if (x_dtype == QRT_F32)
-    route_top_kernel<float><<<grid, block, 0, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top);
+    route_top_kernel<float><<<grid, block, 0, stream>>>((const float*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep);
   else if (x_dtype == QRT_BF16)
-    route_top_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top);
+    route_top_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, router, bias, index, weight, hidden, experts, top, sigmoid_scores, groups, keep);
   else return qrt_fail("route_top: unknown dtype %d", x_dtype);
   QRT_LAUNCH_CHECK("route_top");
   return 0;
@@ -113,7 +154,7 @@ extern "C" int qrt_route_top(const void* x, int x_dtype, const float* router, co
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ gate_up,
                                                           const int* __restrict__ index, T* __restrict__ act,
-                                                          int hidden, int inter, int top) {
+                                                          int hidden, int inter, int top, int act_kind, float limit) {
   extern __shared__ float xs[];  // [hidden]
   const int p = blockIdx.x, t = p / top;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -129,7 +170,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
     if (i >= inter) break;
     const float g = wave_sum(lane_dot<T>(w + (size_t)i * hidden, xs, hidden, lane, wide));
     const float u = wave_sum(lane_dot<T>(w + (size_t)(inter + i) * hidden, xs, hidden, lane, wide));
-    if (lane == 0) act[(size_t)p * inter + i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    if (lane == 0) act[(size_t)p * inter + i] = from_f32<T>(gated_act(g, u, act_kind, limit));
   }
 }
 
@@ -160,8 +201,9 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act
 
 extern "C" int qrt_moe_pairs(const void* x, const void* gate_up, const void* down, const int* index,
                              const float* weight, void* act, float* out, int dtype, int num_tokens, int hidden,
-                             int inter, int experts, int top, hipStream_t stream) {
+                             int inter, int experts, int top, int act_kind, float limit, hipStream_t stream) {
   QRT_CHECK(num_tokens >= 0 && hidden > 0 && inter > 0 && experts > 0 && top > 0, "moe: bad sizes");
+  QRT_CHECK(act_kind == QRT_ACT_SWIGLU || act_kind == QRT_ACT_CLAMPED, "moe: unknown activation %d", act_kind);
   QRT_CHECK((size_t)hidden * 4 <= 64 * 1024 && (size_t)top * inter * 4 <= 64 * 1024,
             "moe: a token's row (%d) or its experts' inner rows (%d x %d) do not fit", hidden, top, inter);
   QRT_CHECK(dtype == QRT_F32 || dtype == QRT_BF16, "moe: unknown dtype %d", dtype);
@@ -170,10 +212,10 @@ extern "C" int qrt_moe_pairs(const void* x, const void* gate_up, const void* dow
   dim3 g1(num_tokens * top, (inter + per_block - 1) / per_block), g2(num_tokens, (hidden + per_block - 1) / per_block);
   QRT_CHECK(g1.y <= 65535 && g2.y <= 65535, "moe: rows too wide for one launch");
   if (dtype == QRT_F32) {
-    moe_gate_up_kernel<float><<<g1, 256, hidden * 4, stream>>>((const float*)x, (const float*)gate_up, index, (float*)act, hidden, inter, top);
+    moe_gate_up_kernel<float><<<g1, 256, hidden * 4, stream>>>((const float*)x, (const float*)gate_up, index, (float*)act, hidden, inter, top, act_kind, limit);
     moe_down_kernel<float><<<g2, 256, top * inter * 4, stream>>>((const float*)act, (const float*)down, index, weight, out, hidden, inter, top);
   } else {
-    moe_gate_up_kernel<bf16_t><<<g1, 256, hidden * 4, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, index, (bf16_t*)act, hidden, inter, top);
+    moe_gate_up_kernel<bf16_t><<<g1, 256, hidden * 4, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, index, (bf16_t*)act, hidden, inter, top, act_kind, limit);
     moe_down_kernel<bf16_t><<<g2, 256, top * inter * 4, stream>>>((const bf16_t*)act, (const bf16_t*)down, index, weight, out, hidden, inter, top);
   }
   QRT_LAUNCH_CHECK("moe_pairs");
@@ -293,7 +335,7 @@ template <typename T, int R, bool GATED>
 __global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __restrict__ in, const T* __restrict__ w,
                                                                  const int* __restrict__ order,
                                                                  const int* __restrict__ offsets, T* __restrict__ out,
-                                                                 int K, int N, int top) {
+                                                                 int K, int N, int top, int act_kind, float limit) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NR = GATED ? 2 * R : R;
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
@@ -342,7 +384,7 @@ __global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __rest
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if (n0 + r >= N) break;
-        if (GATED) out[(size_t)p * N + n0 + r] = from_f32<T>(acc[r] / (1.0f + expf(-acc[r])) * acc[R + r]);
+        if (GATED) out[(size_t)p * N + n0 + r] = from_f32<T>(gated_act(acc[r], acc[R + r], act_kind, limit));
         else out[(size_t)(first + i) * N + n0 + r] = from_f32<T>(acc[r]);
       }
     }
@@ -351,22 +393,22 @@ __global__ __launch_bounds__(256) void moe_rows_by_expert_kernel(const T* __rest
 
 template <typename T, int R, bool GATED>
 static void moe_rows_launch(const void* in, const void* w, const int* order, const int* offsets, void* out, int K, int N,
-                            int experts, int top, hipStream_t stream) {
+                            int experts, int top, int act_kind, float limit, hipStream_t stream) {
   dim3 grid(experts, (N + R - 1) / R);
   const size_t smem = (size_t)(GATED ? 2 * R : R) * K * sizeof(T);
-  moe_rows_by_expert_kernel<T, R, GATED><<<grid, 256, smem, stream>>>((const T*)in, (const T*)w, order, offsets, (T*)out, K, N, top);
+  moe_rows_by_expert_kernel<T, R, GATED><<<grid, 256, smem, stream>>>((const T*)in, (const T*)w, order, offsets, (T*)out, K, N, top, act_kind, limit);
 }
 
 template <typename T, bool GATED>
 static int moe_rows_pick(const void* in, const void* w, const int* order, const int* offsets, void* out, int K, int N,
-                         int experts, int top, hipStream_t stream) {
+                         int experts, int top, int act_kind, float limit, hipStream_t stream) {
   // as many rows a block as 48 KB of LDS hold, eight at most
   const size_t row_bytes = (size_t)(GATED ? 2 : 1) * K * sizeof(T);
   const int fit = (int)(48 * 1024 / row_bytes);
-  if (fit >= 8) moe_rows_launch<T, 8, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
-  else if (fit >= 4) moe_rows_launch<T, 4, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
-  else if (fit >= 2) moe_rows_launch<T, 2, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
-  else if (fit >= 1) moe_rows_launch<T, 1, GATED>(in, w, order, offsets, out, K, N, experts, top, stream);
+  if (fit >= 8) moe_rows_launch<T, 8, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
+  else if (fit >= 4) moe_rows_launch<T, 4, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
+  else if (fit >= 2) moe_rows_launch<T, 2, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
+  else if (fit >= 1) moe_rows_launch<T, 1, GATED>(in, w, order, offsets, out, K, N, experts, top, act_kind, limit, stream);
   else return qrt_fail("moe: rows of %d elements do not fit the block's memory", K);
   return 0;
 }
@@ -374,19 +416,20 @@ static int moe_rows_pick(const void* in, const void* w, const int* order, const 
 // x [T, H] -> act [pairs, I] (by pair) -> y [pairs, H] (by place); order and offsets from qrt_moe_group
 extern "C" int qrt_moe_by_expert(const void* x, const void* gate_up, const void* down, const int* order,
                                  const int* offsets, void* act, void* y, int dtype, int hidden, int inter, int experts,
-                                 int top, hipStream_t stream) {
+                                 int top, int act_kind, float limit, hipStream_t stream) {
   QRT_CHECK(hidden > 0 && inter > 0 && experts >= 1 && experts <= MAX_EXPERTS && top > 0, "moe: bad sizes");
+  QRT_CHECK(act_kind == QRT_ACT_SWIGLU || act_kind == QRT_ACT_CLAMPED, "moe: unknown activation %d", act_kind);
   QRT_CHECK(dtype == QRT_F32 || dtype == QRT_BF16, "moe: unknown dtype %d", dtype);
   const int vec = dtype == QRT_F32 ? 4 : 8;
   QRT_CHECK(hidden % vec == 0 && inter % vec == 0, "moe: widths %d and %d are no multiples of %d", hidden, inter, vec);
   QRT_CHECK((inter + 0) / 1 <= 65535 * 8 && hidden <= 65535 * 8, "moe: rows too many for one launch");
   int rc;
   if (dtype == QRT_F32) {
-    rc = moe_rows_pick<float, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, stream);
-    if (rc == 0) rc = moe_rows_pick<float, false>(act, down, order, offsets, y, inter, hidden, experts, top, stream);
+    rc = moe_rows_pick<float, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream);
+    if (rc == 0) rc = moe_rows_pick<float, false>(act, down, order, offsets, y, inter, hidden, experts, top, act_kind, limit, stream);
   } else {
-    rc = moe_rows_pick<bf16_t, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, stream);
-    if (rc == 0) rc = moe_rows_pick<bf16_t, false>(act, down, order, offsets, y, inter, hidden, experts, top, stream);
+    rc = moe_rows_pick<bf16_t, true>(x, gate_up, order, offsets, act, hidden, inter, experts, top, act_kind, limit, stream);
+    if (rc == 0) rc = moe_rows_pick<bf16_t, false>(act, down, order, offsets, y, inter, hidden, experts, top, act_kind, limit, stream);
   }
   if (rc != 0) return rc;
   QRT_LAUNCH_CHECK("moe_by_expert");

@@ -218,10 +218,7 @@ class DecodeGraph:
                 # now, to choose the length of its pieces by
                 if self.unequal:
                     self.ctx.scratch["attn_lens"] = [runner.cache.length(e.request_id) + 1 for e in entries]
-                self.cache_views = [
-                    None if st.cache is None else runner.cache.view(st.cache, self.ctx.groups, st.writes_cache)
-                    for st in runner.model.plan.order
-                ]
+                self.cache_views = runner.cache.step_views(runner.model.plan.order, self.ctx.groups)
             dev = self.views_dev
             runner.last_row_slots = dev["row_slots"]
             self.runs += 1

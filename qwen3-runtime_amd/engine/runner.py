@@ -158,10 +158,7 @@ class ModelRunner:
 
     def _forward(self, packed: PackedStep, dev: dict[str, torch.Tensor]):
         ctx = self._context(packed, dev)
-        views = [
-            None if st.cache is None else self.cache.view(st.cache, ctx.groups, st.writes_cache)
-            for st in self.model.plan.order
-        ]
+        views = self.cache.step_views(self.model.plan.order, ctx.groups)
         rows = dev["rows"] if packed.num_rows else None
         with torch.inference_mode():
             return self.model.forward(ctx, dev["ids"], views, rows)

@@ -84,6 +84,39 @@ class _AttnTileArgs(Structure):
     ]
 
 
+class _ConvArgs(Structure):
+    _fields_ = [
+        ("x", c_void_p), ("x_stride", c_long), ("taps", c_void_p), ("tail", c_void_p),
+        ("cu_q", c_void_p), ("seq_of_token", c_void_p), ("state_slots", c_void_p), ("out", c_void_p),
+        ("num_tokens", c_int), ("channels", c_int), ("num_taps", c_int), ("nseg", c_int),
+        ("seg_first", c_int * 4), ("seg_heads", c_int * 4), ("seg_width", c_int * 4), ("seg_mode", c_int * 4),
+        ("total_heads", c_int), ("unit_eps", c_float),
+    ]
+
+
+class _RuleArgs(Structure):
+    _fields_ = [
+        ("qkv", c_void_p), ("channels", c_int), ("q_first", c_int), ("k_first", c_int), ("v_first", c_int),
+        ("b", c_void_p), ("b_stride", c_long), ("b_code", c_int),
+        ("a", c_void_p), ("a_stride", c_long), ("a_code", c_int),
+        ("a_log", c_void_p), ("dt_bias", c_void_p), ("state", c_void_p), ("out", c_void_p),
+        ("cu_q", c_void_p), ("state_slots", c_void_p),
+        ("heads", c_int), ("kv_heads", c_int), ("dim", c_int), ("vdim", c_int), ("per_channel", c_int),
+    ]
+
+
+ACTIVATIONS = {"swiglu": 0, "clamped": 1}
+
+
+def _planes(y, t, h, name):
+    """(pointer, dtype code, planes) of a sub-layer output: a matrix [T, H], or float32 planes [P, T, H]."""
+    if y.dim() == 3:
+        _need(y, name, torch.float32, (y.shape[0], t, h))
+        return _ptr(y), F32, y.shape[0]
+    _need(y, name, shape=(t, h))
+    return _ptr(y), _CODE[y.dtype], 1
+
+
 class _SampleArgs(Structure):
     _fields_ = [
         ("logits", c_void_p), ("work", c_void_p), ("counts", c_void_p), ("slot", c_void_p),
@@ -214,7 +247,7 @@ class HipOps:
                                                  c_int(t), c_int(v), c_int(h), _stream()))
         return out
 
-    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, delta_scale=1.0):
         t, h = residual.shape
         _need(residual, "residual", torch.float32)
         _need(weight, "norm weight", torch.float32, (h,))
@@ -233,7 +266,142 @@ class HipOps:
         self._check(self.lib, self.lib.qrt_add_rmsnorm(
             _ptr(residual), _ptr(delta), _CODE[delta.dtype] if delta is not None else F32, _ptr(weight),
             _ptr(rows), _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), c_float(eps), c_int(planes),
-            c_long(plane_stride), _stream()))
+            c_long(plane_stride), c_float(delta_scale), _stream()))
+        return out
+
+    # ---- steps between sub-layers that are neither a product nor a plain norm -----------
+    def norm_mean(self, ya, wa, yb, wb, eps):
+        """``(rmsnorm(ya) * wa + rmsnorm(yb) * wb) / 2`` over the rows, float32 [T, H]; either input a
+        matrix or float32 planes whose sum it is."""
+        t, h = ya.shape[-2:]
+        pa, ca, na = _planes(ya, t, h, "left output")
+        pb, cb, nb = _planes(yb, t, h, "right output")
+        _need(wa, "left weight", torch.float32, (h,))
+        _need(wb, "right weight", torch.float32, (h,))
+        out = torch.empty((t, h), dtype=torch.float32, device=wa.device)
+        self._check(self.lib, self.lib.qrt_norm_mean(pa, c_int(ca), c_int(na), pb, c_int(cb), c_int(nb), _ptr(wa), _ptr(wb),
+                                                     _ptr(out), c_int(t), c_int(h), c_float(eps), _stream()))
+        return out
+
+    def add_concat(self, residual, delta, delta_scale, origin, out_dtype):
+        """``[residual + delta_scale * delta | origin]``, [T, 2H] in ``out_dtype``."""
+        t, h = residual.shape
+        _need(residual, "residual", torch.float32)
+        _need(origin, "origin", torch.float32, (t, h))
+        pd, cd, nd = (None, F32, 1) if delta is None else _planes(delta, t, h, "delta")
+        out = torch.empty((t, 2 * h), dtype=out_dtype, device=residual.device)
+        self._check(self.lib, self.lib.qrt_add_concat(_ptr(residual), pd, c_int(cd), c_int(nd), c_float(delta_scale),
+                                                      _ptr(origin), _ptr(out), _CODE[out_dtype], c_int(t), c_int(h), _stream()))
+        return out
+
+    def accumulate(self, acc, y):
+        """``acc += y`` (float32 [T, H]; ``y`` a matrix or planes); returns ``acc``."""
+        t, h = acc.shape
+        _need(acc, "sum", torch.float32)
+        py, cy, ny = _planes(y, t, h, "addend")
+        self._check(self.lib, self.lib.qrt_accumulate(_ptr(acc), py, c_int(cy), c_int(ny), c_long(t * h), _stream()))
+        return acc
+
+    def gated_act(self, gate_up, activation="swiglu", limit=0.0):
+        """The gated activation of [T, 2I] (gate columns first): ``swiglu``, or ``clamped``."""
+        if activation == "swiglu":
+            return self.swiglu(gate_up)
+        _need(gate_up, "gate_up")
+        t, two_i = gate_up.shape
+        if two_i % 2:
+            raise OpsError(f"gate_up has odd width {two_i}")
+        out = torch.empty((t, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+        self._check(self.lib, self.lib.qrt_gated_act(_ptr(gate_up), _ptr(out), _CODE[gate_up.dtype], c_int(t),
+                                                     c_int(two_i // 2), c_int(ACTIVATIONS[activation]), c_float(limit), _stream()))
+        return out
+
+    def bias_rotate_pairs(self, x, bias, positions, freq, rot_heads, head_dim):
+        """In place on a product's output [T, W]: add ``bias`` [W] (float32; None: none), then turn
+        the first ``2 * len(freq)`` elements of each of the first ``rot_heads`` heads of ``head_dim``
+        columns, in interleaved pairs, by ``positions * freq`` (``freq`` None: no rotation)."""
+        t, w = x.shape
+        _need(x, "x")
+        if bias is not None:
+            _need(bias, "bias", torch.float32, (w,))
+        pairs = 0
+        if freq is not None:
+            pairs = freq.numel()
+            _need(freq, "freq", torch.float32, (pairs,))
+            _need(positions, "positions", torch.int32, (t,))
+        self._check(self.lib, self.lib.qrt_bias_rotate_pairs(_ptr(x), c_long(x.stride(0)), c_int(w), _CODE[x.dtype], _ptr(bias),
+                                                             _ptr(positions) if freq is not None else None, _ptr(freq),
+                                                             c_int(rot_heads), c_int(head_dim), c_int(pairs), c_int(t), _stream()))
+        return x
+
+    # ---- gated delta rule ---------------------------------------------------------------
+    def delta_conv(self, ctx, y, channels, taps, tail, segments, unit_eps):
+        """The first ``channels`` columns of ``y`` [T, W] through their causal convolutions
+        (``taps`` float32 [C, K]) and silu, then per head as ``segments`` say, each (heads, width,
+        mode): 0 as it is, 1 scaled to a unit vector, 2 that times width^(-1/2). float32 [T, C].
+        ``tail`` [slots, C, K-1] float32 holds each request's last inputs and is brought up to date."""
+        t, w = y.shape
+        _need(y, "projections")
+        k = taps.shape[1]
+        _need(taps, "taps", torch.float32, (channels, k))
+        slots = tail.shape[0]
+        _need(tail, "convolution tail", torch.float32, (slots, channels, max(k - 1, 1)))
+        if t != ctx.num_tokens or channels > w or not 1 <= len(segments) <= 4:
+            raise OpsError(f"delta_conv: {t} rows for {ctx.num_tokens} tokens, {channels} channels in {w} columns")
+        a = _ConvArgs()
+        a.x, a.x_stride, a.taps, a.tail = y.data_ptr(), y.stride(0), taps.data_ptr(), tail.data_ptr()
+        a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
+        a.seq_of_token = _need(ctx.seq_of_token, "seq_of_token", torch.int32, (t,)).data_ptr()
+        a.state_slots = _need(ctx.state_slots, "state_slots", torch.int32, (ctx.num_seqs,)).data_ptr()
+        out = torch.empty((t, channels), dtype=torch.float32, device=y.device)
+        a.out, a.num_tokens, a.channels, a.num_taps, a.nseg, a.unit_eps = out.data_ptr(), t, channels, k, len(segments), unit_eps
+        first = 0
+        for i, (heads, width, mode) in enumerate(segments):
+            a.seg_first[i], a.seg_heads[i], a.seg_width[i], a.seg_mode[i] = first, heads, width, mode
+            first += heads * width
+        if first != channels:
+            raise OpsError(f"delta_conv: segments cover {first} of {channels} channels")
+        self._check(self.lib, self.lib.qrt_delta_conv(byref(a), _CODE[y.dtype], c_int(ctx.num_seqs), c_int(slots), _stream()))
+        return out
+
+    def delta_rule(self, ctx, qkv, beta, a_logits, a_log, dt_bias, state, heads, kv_heads, dim, vdim, per_channel):
+        """The recurrence over each sequence's tokens from its slot's state (float32
+        [slots, heads, vdim, dim], updated in place). ``qkv`` float32 [T, C] as ``delta_conv`` leaves
+        it; ``beta`` [T, heads] and ``a_logits`` [T, heads] (or [T, heads * dim], ``per_channel``)
+        may be columns of wider matrices. Returns the read-outs, float32 [T, heads, vdim]."""
+        t = ctx.num_tokens
+        c = 2 * kv_heads * dim + heads * vdim
+        _need(qkv, "convolved q | k | v", torch.float32, (t, c))
+        _need(state, "state", torch.float32, (state.shape[0], heads, vdim, dim))
+        per = heads * dim if per_channel else heads
+        for name, m, width in (("beta", beta, heads), ("decay logits", a_logits, per)):
+            if not m.is_cuda or tuple(m.shape) != (t, width) or m.stride(1) != 1 or m.dtype not in _CODE:
+                raise OpsError(f"{name}: {tuple(m.shape)} {m.dtype} with strides {m.stride()} for {t} tokens of {width}")
+        _need(a_log, "A_log", torch.float32, (heads,))
+        _need(dt_bias, "dt_bias", torch.float32, (per,))
+        a = _RuleArgs()
+        a.qkv, a.channels, a.q_first, a.k_first, a.v_first = qkv.data_ptr(), c, 0, kv_heads * dim, 2 * kv_heads * dim
+        a.b, a.b_stride, a.b_code = beta.data_ptr(), beta.stride(0), _CODE[beta.dtype]
+        a.a, a.a_stride, a.a_code = a_logits.data_ptr(), a_logits.stride(0), _CODE[a_logits.dtype]
+        a.a_log, a.dt_bias, a.state = a_log.data_ptr(), dt_bias.data_ptr(), state.data_ptr()
+        out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qkv.device)
+        a.out = out.data_ptr()
+        a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
+        a.state_slots = _need(ctx.state_slots, "state_slots", torch.int32, (ctx.num_seqs,)).data_ptr()
+        a.heads, a.kv_heads, a.dim, a.vdim, a.per_channel = heads, kv_heads, dim, vdim, int(bool(per_channel))
+        self._check(self.lib, self.lib.qrt_delta_rule(byref(a), c_int(t), c_int(ctx.num_seqs), _stream()))
+        return out
+
+    def delta_out(self, o, weight, gate, eps, gate_kind, out_dtype):
+        """Per head: ``o / rms(o) * weight * act(gate)``, act silu or sigmoid; [T, heads * vdim]."""
+        t, heads, vdim = o.shape
+        _need(o, "read-out", torch.float32)
+        _need(weight, "read-out norm weight", torch.float32, (vdim,))
+        if not gate.is_cuda or tuple(gate.shape) != (t, heads * vdim) or gate.stride(1) != 1 or gate.dtype not in _CODE:
+            raise OpsError(f"gate {tuple(gate.shape)} {gate.dtype} does not fit {t} tokens of {heads} heads of {vdim}")
+        out = torch.empty((t, heads * vdim), dtype=out_dtype, device=o.device)
+        self._check(self.lib, self.lib.qrt_delta_out(_ptr(o), _ptr(weight), c_void_p(gate.data_ptr()), c_long(gate.stride(0)),
+                                                     _CODE[gate.dtype], _ptr(out), _CODE[out_dtype], c_int(t), c_int(heads),
+                                                     c_int(vdim), c_float(eps), c_int({"silu": 0, "sigmoid": 1}[gate_kind]), _stream()))
         return out
 
     def mix_norm(self, streams, update, read, weight, bias, eps, out_dtype, rows=None):
@@ -278,9 +446,12 @@ class HipOps:
         return out
 
     # ---- routed experts --------------------------------------------------------------
-    def route_top(self, x, router, router_bias, top):
+    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None):
         """Router logits ``x W^T + b`` in float32, the ``top`` largest per token and the softmax
-        over those alone: (int32 [T, top], float32 [T, top])."""
+        over those alone: (int32 [T, top], float32 [T, top]). ``scoring="sigmoid"``: the choice goes
+        by ``sigmoid`` of the logits, which are also the weights, as they are. ``groups``, ``keep``:
+        only experts of the ``keep`` best of ``groups`` equal groups of neighbours can be chosen, a
+        group's score being the sum of its two largest entries."""
         t, h = x.shape
         _need(x, "x")
         n = router.shape[0]
@@ -291,10 +462,11 @@ class HipOps:
         weight = torch.empty((t, top), dtype=torch.float32, device=x.device)
         self._check(self.lib, self.lib.qrt_route_top(_ptr(x), _CODE[x.dtype], _ptr(router), _ptr(router_bias),
                                                      _ptr(index), _ptr(weight), c_int(t), c_int(h), c_int(n),
-                                                     c_int(top), _stream()))
+                                                     c_int(top), c_int(scoring == "sigmoid"), c_int(groups),
+                                                     c_int(groups if keep is None else keep), _stream()))
         return index, weight
 
-    def moe_swiglu(self, x, gate_up, down, index, weight):
+    def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0):
         """``sum_j weight[t, j] * down[e] (silu(gate[e] x) * (up[e] x))`` with ``e = index[t, j]``;
         ``gate_up`` [E, 2I, H] (gate rows first), ``down`` [E, H, I]. float32 [T, H]."""
         t, h = x.shape
@@ -312,7 +484,8 @@ class HipOps:
         pairs = t * top
         if (pairs >= self.moe_grouped_min_pairs and pairs >= self.moe_grouped_pairs_per_expert * n
                 and not torch.cuda.is_current_stream_capturing()):
-            return self._moe_grouped(x, gate_up, down, index, weight, out)
+            return self._moe_grouped(x, gate_up, down, index, weight, out, activation, limit)
+        kind = (c_int(ACTIVATIONS[activation]), c_float(limit))
         act = torch.empty((t * top, inter), dtype=x.dtype, device=x.device)
         vec = 16 // x.element_size()
         if pairs >= self.moe_by_expert_pairs_per_expert * n and h % vec == 0 and inter % vec == 0:
@@ -325,14 +498,14 @@ class HipOps:
                                                          c_int(pairs), c_int(n), _stream()))
             self._check(self.lib, self.lib.qrt_moe_by_expert(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(order), _ptr(offsets),
                                                              _ptr(act), _ptr(y), _CODE[x.dtype], c_int(h), c_int(inter),
-                                                             c_int(n), c_int(top), _stream()))
+                                                             c_int(n), c_int(top), *kind, _stream()))
             self._check(self.lib, self.lib.qrt_moe_combine(_ptr(y), _ptr(place), _ptr(index), _ptr(offsets), c_int(0),
                                                            _ptr(weight), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
                                                            c_int(top), _stream()))
             return out
         self._check(self.lib, self.lib.qrt_moe_pairs(_ptr(x), _ptr(gate_up), _ptr(down), _ptr(index), _ptr(weight),
                                                      _ptr(act), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
-                                                     c_int(inter), c_int(n), c_int(top), _stream()))
+                                                     c_int(inter), c_int(n), c_int(top), *kind, _stream()))
         return out
 
     # Steps of many tokens run the experts one by one, each on the rows of its own tokens, with
@@ -346,7 +519,7 @@ class HipOps:
     # walks the expert's tokens; below it, once per pair (fewer launches, and pairs rarely meet).
     moe_by_expert_pairs_per_expert = 1
 
-    def _moe_grouped(self, x, gate_up, down, index, weight, out):
+    def _moe_grouped(self, x, gate_up, down, index, weight, out, activation="swiglu", limit=0.0):
         t, h = x.shape
         n, top = gate_up.shape[0], index.shape[1]
         pairs = t * top
@@ -379,7 +552,7 @@ class HipOps:
                     torch.mm(xs[a:b], gate_up[e].t(), out=both[a:b])
                 else:
                     both[a:b] = self.linear(xs[a:b], gate_up[e])
-            act = self.swiglu(both)
+            act = self.gated_act(both, activation, limit)
             for e, a, b in busy:
                 if b - a > self.own_max_rows:
                     torch.mm(act[a:b], down[e].t(), out=y[a:b])
@@ -387,7 +560,7 @@ class HipOps:
                     y[a:b] = self.linear(act[a:b], down[e])
         else:
             for e, a, b in busy:
-                y[a:b] = self.linear(self.gated_linear(xs[a:b], gate_up[e]), down[e])
+                y[a:b] = self.linear(self.gated_linear(xs[a:b], gate_up[e], activation, limit), down[e])
         self._check(self.lib, self.lib.qrt_moe_combine(_ptr(y), _ptr(place), _ptr(index), _ptr(offsets), c_int(padded),
                                                        _ptr(weight), _ptr(out), _CODE[x.dtype], c_int(t), c_int(h),
                                                        c_int(top), _stream()))
@@ -538,7 +711,7 @@ class HipOps:
         return max(1, min(8, 256 // blocks, (k // 32) // 12))
 
 
-    def gated_linear(self, x, w_gate_up):
+    def gated_linear(self, x, w_gate_up, activation="swiglu", limit=0.0):
         """``swiglu(linear(x, w_gate_up))`` with ``w_gate_up`` [2I, K], gate rows first. With few
         rows in bfloat16 one kernel forms both halves and applies the activation in its epilogue,
         so the [T, 2I] intermediate never reaches memory."""
@@ -546,6 +719,8 @@ class HipOps:
         two_i, kw = w_gate_up.shape
         if k != kw or two_i % 2:
             raise OpsError(f"gated_linear: x is {tuple(x.shape)}, weight is {tuple(w_gate_up.shape)}")
+        if activation != "swiglu":  # the products' fused epilogue is SwiGLU's
+            return self.gated_act(self.linear(x, w_gate_up), activation, limit)
         if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and k % 32 == 0:
             _need(x, "x")
             _need(w_gate_up, "weight")

@@ -1,6 +1,6 @@
 """Layer parts. Importing this package registers the shipped kinds."""
 
-from . import attention, block, embedding, mlp, moe, norm, rope  # noqa: F401
+from . import attention, block, delta, embedding, entry, mlp, moe, norm, parallel, rope  # noqa: F401
 from .base import (  # noqa: F401
     Block,
     CacheView,

@@ -17,7 +17,9 @@ by their root mean square); a fixed score ``scale``; a cap on the scaled scores,
 ``softcap * tanh(score / softcap)``, before the softmax; a mask of chunks instead of a window
 (``chunk``: key ``j`` is visible iff ``j <= i`` and ``j // chunk == i // chunk``, chunks counted
 from position 0 of the sequence); an output gate (``output_gate``: one more projection ``g`` of
-the mixer's input, whose sigmoid multiplies the concatenated heads before the output projection).
+the mixer's input, whose sigmoid multiplies the concatenated heads before the output projection);
+biases on the q, k and v projections (``bias``: tensors ``q_bias``, ``k_bias``, ``v_bias``, added to the
+product's output in float32, before any rotation).
 """
 
 from __future__ import annotations
@@ -48,6 +50,7 @@ class GroupedQueryAttention(Mixer):
         softcap: float | None = None,
         chunk: int | None = None,
         output_gate: bool = False,
+        bias: bool = False,
         tensors=None,
     ):
         super().__init__(tensors)
@@ -66,6 +69,8 @@ class GroupedQueryAttention(Mixer):
         self.qk_norm_weight = bool(qk_norm_weight)
         self.softcap = None if softcap is None else float(softcap)
         self.output_gate = bool(output_gate)
+        self.has_bias = bool(bias)
+        self.bias = None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = None
         if position is not None:
@@ -89,6 +94,10 @@ class GroupedQueryAttention(Mixer):
         ]
         if self.output_gate:
             decls.append(TensorDecl(self._name("g"), (self.num_heads * dv, h)))
+        if self.has_bias:
+            decls += [TensorDecl(self._name("q_bias"), (self.num_heads * d,)),
+                      TensorDecl(self._name("k_bias"), (self.num_kv_heads * d,)),
+                      TensorDecl(self._name("v_bias"), (self.num_kv_heads * dv,))]
         if self.qk_norm_eps is not None and self.qk_norm_weight:
             decls += [
                 TensorDecl(self._name("q_norm"), (d,), init="norm"),
@@ -101,6 +110,11 @@ class GroupedQueryAttention(Mixer):
         names = [self._name("q"), self._name("k"), self._name("v")] + ([self._name("g")] if self.output_gate else [])
         self.qkv = fetch.fused(names, dim=0)
         self.o = fetch.matrix(self._name("o"))
+        if self.has_bias:  # one vector over the product's columns; a gate's columns get zeros
+            pieces = [fetch.vector_f32(self._name(n)) for n in ("q_bias", "k_bias", "v_bias")]
+            if self.output_gate:
+                pieces.append(torch.zeros(self.num_heads * self.value_dim, dtype=torch.float32, device=pieces[0].device))
+            self.bias = fetch.constant(torch.cat(pieces))
         if self.qk_norm_eps is not None and self.qk_norm_weight:
             self.q_norm = fetch.vector_f32(self._name("q_norm"))
             self.k_norm = fetch.vector_f32(self._name("k_norm"))
@@ -125,8 +139,17 @@ class GroupedQueryAttention(Mixer):
         nq, nkv, d, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
         qkv = ops.linear(x, self.qkv)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        fused = self.position is None or self.position.fused_form == "neox_full"
-        inv_freq = None if self.position is None or not fused else self.position.inv_freq
+        in_place = getattr(self.position, "in_place", False)
+        if in_place:
+            # biases and an encoding that works on the product where it lies: after it the mixer
+            # goes on as one without encoding
+            if self.qk_norm_eps is not None:
+                raise NotImplementedError("a q/k norm in front of an encoding that works in place")
+            self.position.rotate_in_place(ctx, qkv, nq + nkv, self.bias)
+        elif self.bias is not None:
+            ops.bias_rotate_pairs(qkv, self.bias, ctx.positions, None, 0, d)
+        fused = self.position is None or in_place or self.position.fused_form == "neox_full"
+        inv_freq = None if self.position is None or in_place or not fused else self.position.inv_freq
         # what only some designs have travels by name, and only where it is set
         more = {}
         if dv != d:
@@ -143,7 +166,7 @@ class GroupedQueryAttention(Mixer):
             # a step of single tokens: all of it inside the attention kernel
             attn = ops.decode_attention(qkv, cache, ctx, nq, nkv, d, self.scale, self.window,
                                         self.q_norm, self.k_norm, eps, inv_freq,
-                                        None if self.position is None else self.position.angles_key, **more)
+                                        None if inv_freq is None else self.position.angles_key, **more)
             return ops.linear_for_residual(attn, self.o)
         if fused:
             # norm, rotation and the cache write in one pass over qkv
@@ -153,7 +176,7 @@ class GroupedQueryAttention(Mixer):
             q = ops.qk_norm_rope_store(
                 qkv, nq, nkv, d, self.q_norm, self.k_norm, eps, inv_freq, ctx.positions,
                 cache if cache.writes else None, ctx=ctx,
-                angles_key=None if self.position is None else self.position.angles_key, **shape,
+                angles_key=None if inv_freq is None else self.position.angles_key, **shape,
             )
         elif dv != d or gate_width:
             raise NotImplementedError("a position encoding without a fused form, with values of another size "

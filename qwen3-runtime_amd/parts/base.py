@@ -16,6 +16,8 @@ Roles and the call each must answer (``T`` tokens of this step, ``H`` width):
 * feed_forward   ``forward(ctx, x[T, H]) -> [T, H]``
 * position       ``rotate(ctx, q[T, nq, D], k[T, nkv, D]) -> (q, k)``
 * block          ``forward(ctx, residual, delta, cache) -> (residual, delta)``
+* entry          ``forward(ctx, residual, delta, origin) -> (residual, delta)``; ``origin`` is the
+                 embedding's output [T, H] float32, which no part changes
 * head           ``forward(ctx, x[R, H]) -> logits[R, V] float32``
 
 The residual stream is float32 in every mode; ``delta`` is the output of the
@@ -124,6 +126,13 @@ class Mixer(Part):
     def cache_spec(self) -> CacheSpec | None:
         return None
 
+    def cache_specs(self) -> tuple[CacheSpec, ...]:
+        """Everything the mixer keeps between steps. One thing or none: what ``cache_spec`` says,
+        and ``forward`` gets one ``CacheView`` (or None). A mixer that keeps several overrides
+        this, and its ``forward`` gets a tuple of views in the same order."""
+        spec = self.cache_spec()
+        return () if spec is None else (spec,)
+
 
 class FeedForward(Part):
     role = "feed_forward"
@@ -148,6 +157,10 @@ class PositionEncoding(Part):
 
 class Block(Part):
     role = "block"
+
+
+class Entry(Part):
+    role = "entry"
 
 
 @dataclass

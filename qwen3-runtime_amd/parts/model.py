@@ -41,25 +41,31 @@ class DecoderModel:
             )
         self.final_norm = build_part("norm", plan.final_norm)
         self.head = build_part("head", plan.head)
+        self.entries = [build_part("entry", spec) for spec in plan.entries]
         self._check_caches()
 
     def _check_caches(self) -> None:
         for i, step in enumerate(self.plan.order):
-            spec = self.blocks[step.layer].mixer.cache_spec()
-            if spec is None:
-                if step.cache is not None:
+            specs = self.blocks[step.layer].mixer.cache_specs()
+            ids = step.cache_ids()
+            if not specs:
+                if ids:
                     raise ValueError(f"order[{i}]: layer {step.layer}'s mixer keeps no cache")
                 continue
-            if step.cache is None:
-                raise ValueError(f"order[{i}]: layer {step.layer}'s mixer needs a cache")
-            have = self.plan.caches[step.cache]
-            if have.group_key() != spec.group_key():
-                raise ValueError(
-                    f"order[{i}]: layer {step.layer} needs cache {spec}, the plan gives {have}"
-                )
+            if len(ids) != len(specs):
+                raise ValueError(f"order[{i}]: layer {step.layer}'s mixer needs {len(specs)} cache(s), "
+                                 f"the plan names {len(ids)}")
+            for cache, spec in zip(ids, specs):
+                have = self.plan.caches[cache]
+                if have.group_key() != spec.group_key():
+                    raise ValueError(
+                        f"order[{i}]: layer {step.layer} needs cache {spec}, the plan gives {have}"
+                    )
 
     def parts(self):
         yield from walk(self.embedding)
+        for entry in self.entries:
+            yield from walk(entry)
         for block in self.blocks:
             yield from walk(block)
         yield from walk(self.final_norm)
@@ -79,7 +85,10 @@ class DecoderModel:
         """Bytes of weights and floating-point operations of one step (``Part.step_cost``), summed
         over the parts in the order they run: a layer named twice computes twice and is read once."""
         cost = StepCost()
-        runs = [self.embedding] + [self.blocks[step.layer] for step in self.plan.order] + [self.final_norm, self.head]
+        runs = [self.embedding]
+        for step in self.plan.order:
+            runs += ([self.entries[step.entry]] if step.entry is not None else []) + [self.blocks[step.layer]]
+        runs += [self.final_norm, self.head]
         for top in runs:
             for part in walk(top):
                 cost.add(part.step_cost(spans, rows, elem_bytes))
@@ -103,7 +112,8 @@ class DecoderModel:
             part.load(fetch)
 
     def forward(self, ctx: StepContext, ids, caches: Sequence[CacheView | None], rows=None):
-        """``ids`` int32 [T]; ``caches[i]`` is the view for ``plan.order[i]``.
+        """``ids`` int32 [T]; ``caches[i]`` is the view for ``plan.order[i]`` (a tuple of views for
+        a step that names several caches).
 
         Returns logits ``[R, V]`` float32 for the packed row indices ``rows``
         (int32 tensor), or None when ``rows`` is None: the pass then only fills
@@ -112,7 +122,11 @@ class DecoderModel:
         ctx.per_pass.clear()
         residual = self.embedding.forward(ctx, ids)
         delta = None
+        # entries read the embedding's output; the stream itself is updated in place, so they get a copy
+        origin = residual.clone() if self.entries else None
         for step, cache in zip(self.plan.order, caches):
+            if step.entry is not None:
+                residual, delta = self.entries[step.entry].forward(ctx, residual, delta, origin)
             residual, delta = self.blocks[step.layer].forward(ctx, residual, delta, cache)
         if rows is None:
             return None

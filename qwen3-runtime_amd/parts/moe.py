@@ -1,4 +1,4 @@
-"""Routed mixture of SwiGLU experts.
+"""Routed mixture of gated experts.
 
 A router scores every token against ``num_experts`` experts in float32 (``z = W_r h + b_r``);
 the token takes the ``top`` experts with the largest logits, weighted by the softmax over
@@ -6,6 +6,15 @@ those logits alone, and the output is the weighted sum of the chosen experts' ou
 ``down_e( silu(gate_e(x)) * up_e(x) )``. Experts have no biases. On the device all experts'
 matrices lie in two tensors, ``[E, 2I, H]`` (gate rows, then up rows) and ``[E, H, I]``, so that
 one launch serves every (token, chosen expert) pair.
+
+Options beyond that form. ``scoring="sigmoid"``: scores ``s = sigmoid(z)``; the ``top`` largest are
+chosen and weigh the experts' outputs as they are, not renormalised. ``groups`` and ``keep``: the
+experts form ``groups`` equal groups of neighbours, a group's score is the sum of its two largest
+scores, and only experts of the ``keep`` best groups can be chosen. ``activation="clamped"`` with
+``limit``: ``g = min(gate x, limit)``, ``u = clamp(up x, -limit, limit)``, ``y = g sigmoid(1.702 g) (u + 1)``
+in place of ``silu(g) u``. ``shared_size``: one more expert of that inner width (tensors
+``shared_gate``, ``shared_up``, ``shared_down``; ``shared_limit`` its clamp) that every token passes
+and whose output is added unweighted.
 """
 
 from __future__ import annotations
@@ -15,13 +24,16 @@ from .base import FeedForward, StepCost
 from .plan import TensorDecl
 
 
+@register_part("feed_forward", "routed_experts")
 @register_part("feed_forward", "moe_swiglu")
 class RoutedSwiGLU(FeedForward):
     """``tensors``: ``router``, ``router_bias`` (with ``router_bias=True``), and ``gate``, ``up``,
     ``down`` as patterns in which ``{e}`` stands for the expert's number."""
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
-                 router_bias: bool = True, tensors=None):
+                 router_bias: bool = True, scoring: str = "softmax_top", groups: int = 1, keep: int | None = None,
+                 activation: str = "swiglu", limit: float = 0.0, shared_size: int | None = None,
+                 shared_limit: float | None = None, tensors=None):
         super().__init__(tensors)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
@@ -30,7 +42,19 @@ class RoutedSwiGLU(FeedForward):
         if not 1 <= self.top <= self.num_experts:
             raise ValueError(f"each token takes {self.top} of {self.num_experts} experts")
         self.has_router_bias = bool(router_bias)
+        if scoring not in ("softmax_top", "sigmoid") or activation not in ("swiglu", "clamped"):
+            raise ValueError(f"unknown scoring {scoring!r} (softmax_top, sigmoid) or activation {activation!r} (swiglu, clamped)")
+        self.scoring, self.activation, self.limit = scoring, activation, float(limit)
+        self.groups = int(groups)
+        self.keep = self.groups if keep is None else int(keep)
+        if self.groups < 1 or self.num_experts % self.groups or not 1 <= self.keep <= self.groups:
+            raise ValueError(f"{self.num_experts} experts in {self.groups} groups of which {self.keep} stay")
+        if self.keep * (self.num_experts // self.groups) < self.top:
+            raise ValueError(f"{self.keep} groups of {self.num_experts // self.groups} experts hold fewer than the {self.top} chosen")
+        self.shared_size = None if shared_size is None else int(shared_size)
+        self.shared_limit = self.limit if shared_limit is None else float(shared_limit)
         self.router = self.router_bias = self.gate_up = self.down = None
+        self.shared_gate_up = self.shared_down = None
 
     def _expert(self, logical: str, e: int) -> str:
         return self._name(logical).format(e=e)
@@ -43,6 +67,10 @@ class RoutedSwiGLU(FeedForward):
         for e in range(self.num_experts):
             decls += [TensorDecl(self._expert("gate", e), (i, h)), TensorDecl(self._expert("up", e), (i, h)),
                       TensorDecl(self._expert("down", e), (h, i))]
+        if self.shared_size:
+            s = self.shared_size
+            decls += [TensorDecl(self._name("shared_gate"), (s, h)), TensorDecl(self._name("shared_up"), (s, h)),
+                      TensorDecl(self._name("shared_down"), (h, s))]
         return decls
 
     def load(self, fetch):
@@ -54,6 +82,9 @@ class RoutedSwiGLU(FeedForward):
         names = [self._expert(part, e) for e in range(n) for part in ("gate", "up")]
         self.gate_up = fetch.fused(names, dim=0).view(n, 2 * i, h)
         self.down = fetch.fused([self._expert("down", e) for e in range(n)], dim=0).view(n, h, i)
+        if self.shared_size:
+            self.shared_gate_up = fetch.fused([self._name("shared_gate"), self._name("shared_up")], dim=0)
+            self.shared_down = fetch.matrix(self._name("shared_down"))
 
     def step_cost(self, spans, rows, elem_bytes):
         # only the experts that some token chose are read, and each token multiplies `top` of them
@@ -66,8 +97,23 @@ class RoutedSwiGLU(FeedForward):
             for part, size in (("gate", i * h), ("up", i * h), ("down", h * i)):
                 cost.weight_bytes[self._expert(part, e)] = size * elem_bytes
         cost.flop = 2.0 * tokens * (n * h + self.top * 3 * h * i)
+        if self.shared_size:
+            for part in ("shared_gate", "shared_up", "shared_down"):
+                cost.weight_bytes[self._name(part)] = self.shared_size * h * elem_bytes
+            cost.flop += 2.0 * tokens * 3 * h * self.shared_size
         return cost
 
     def forward(self, ctx, x):
-        index, weight = ctx.ops.route_top(x, self.router, self.router_bias, self.top)
-        return ctx.ops.moe_swiglu(x, self.gate_up, self.down, index, weight)
+        ops = ctx.ops
+        plain = self.scoring == "softmax_top" and self.groups == 1 and self.activation == "swiglu"
+        if plain:
+            index, weight = ops.route_top(x, self.router, self.router_bias, self.top)
+            out = ops.moe_swiglu(x, self.gate_up, self.down, index, weight)
+        else:
+            index, weight = ops.route_top(x, self.router, self.router_bias, self.top, scoring=self.scoring,
+                                          groups=self.groups, keep=self.keep)
+            out = ops.moe_swiglu(x, self.gate_up, self.down, index, weight, activation=self.activation, limit=self.limit)
+        if self.shared_size:
+            act = ops.gated_linear(x, self.shared_gate_up, activation=self.activation, limit=self.shared_limit)
+            out = ops.accumulate(out, ops.linear_for_residual(act, self.shared_down))
+        return out

@@ -1,7 +1,8 @@
 """Norms with the residual update fused in front of them.
 
 ``rmsnorm``: ``y = x * rsqrt(mean(x^2) + eps) * w`` over the last dimension, all in
-float32, the weight multiplying after normalisation, no offset, no bias
+float32, the weight multiplying after normalisation, no offset, no bias; with ``delta_scale``
+the pending output joins the stream as ``x + delta_scale * delta``
 (reference: qwen3_runtime/layers/ops.py:17-20). The fused form first adds the
 pending sub-layer output into the residual stream
 (reference: qwen3_runtime/layers/ops.py:28-37), here in float32.
@@ -29,12 +30,16 @@ from .plan import TensorDecl
 class RMSNorm(Norm):
     has_bias = False
 
-    def __init__(self, size: int, eps: float, streams: int = 1, tensors=None):
+    def __init__(self, size: int, eps: float, streams: int = 1, delta_scale: float = 1.0, tensors=None):
         super().__init__(tensors)
         self.size = int(size)
         self.eps = float(eps)
         self.streams = int(streams)
         self.weight = self.bias = self.read_all = None
+        # what multiplies a pending sub-layer output as it joins the stream (1: the plain sum)
+        self.delta_scale = float(delta_scale)
+        if self.delta_scale != 1.0 and (self.streams > 1 or self.has_bias):
+            raise ValueError("a scaled residual sum goes with the RMS norm over one stream")
 
     def tensor_decls(self):
         decls = [TensorDecl(self._name("weight"), (self.size,), init="norm")]
@@ -60,6 +65,8 @@ class RMSNorm(Norm):
                                     self.bias, self.eps, ctx.dtype, rows)
         if self.has_bias:
             return ctx.ops.mix_norm(residual, delta, None, self.weight, self.bias, self.eps, ctx.dtype, rows)
+        if self.delta_scale != 1.0:
+            return ctx.ops.add_rmsnorm(residual, delta, self.weight, self.eps, ctx.dtype, rows, delta_scale=self.delta_scale)
         return ctx.ops.add_rmsnorm(residual, delta, self.weight, self.eps, ctx.dtype, rows)
 
 

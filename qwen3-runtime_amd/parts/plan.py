@@ -140,13 +140,23 @@ class RunStep:
     """One entry of the execution order.
 
     ``layer`` indexes ``ModelPlan.layers``. ``cache`` indexes ``ModelPlan.caches``
-    (or is None for a mixer without cache). ``writes_cache`` is False when the
-    step only reads a cache that an earlier step of the same pass wrote.
+    (or is None for a mixer without cache); a mixer that keeps several things (pages of keys
+    and a recurrent state, say) names them all, as a tuple in the order of its
+    ``cache_specs()``, and its ``forward`` receives as many views. ``writes_cache`` is False
+    when the step only reads a cache that an earlier step of the same pass wrote.
+    ``entry`` indexes ``ModelPlan.entries``: a part that works on the residual stream right
+    before this step's layer (the start of a pass over a looped span, say).
     """
 
     layer: int
-    cache: int | None = None
+    cache: int | tuple[int, ...] | None = None
     writes_cache: bool = True
+    entry: int | None = None
+
+    def cache_ids(self) -> tuple[int, ...]:
+        if self.cache is None:
+            return ()
+        return tuple(self.cache) if isinstance(self.cache, (tuple, list)) else (self.cache,)
 
 
 @dataclass(frozen=True)
@@ -163,19 +173,22 @@ class ModelPlan:
     # tensors a model file may hold although the plan reads them from elsewhere
     ignorable: Sequence[str] = ()
     eos_token_id: int | None = None
+    # parts of role "entry" that steps of the order may name (``RunStep.entry``)
+    entries: Sequence[PartSpec] = ()
 
     def __post_init__(self) -> None:
         writers: set[int] = set()
         for i, step in enumerate(self.order):
             if not 0 <= step.layer < len(self.layers):
                 raise ValueError(f"order[{i}] names layer {step.layer}; the plan has {len(self.layers)}")
-            if step.cache is None:
-                continue
-            if not 0 <= step.cache < len(self.caches):
-                raise ValueError(f"order[{i}] names cache {step.cache}; the plan has {len(self.caches)}")
-            if step.writes_cache:
-                if step.cache in writers:
-                    raise ValueError(f"cache {step.cache} is written by two steps of the order")
-                writers.add(step.cache)
-            elif step.cache not in writers:
-                raise ValueError(f"order[{i}] reads cache {step.cache} before any step writes it")
+            if step.entry is not None and not 0 <= step.entry < len(self.entries):
+                raise ValueError(f"order[{i}] names entry {step.entry}; the plan has {len(self.entries)}")
+            for cache in step.cache_ids():
+                if not 0 <= cache < len(self.caches):
+                    raise ValueError(f"order[{i}] names cache {cache}; the plan has {len(self.caches)}")
+                if step.writes_cache:
+                    if cache in writers:
+                        raise ValueError(f"cache {cache} is written by two steps of the order")
+                    writers.add(cache)
+                elif cache not in writers:
+                    raise ValueError(f"order[{i}] reads cache {cache} before any step writes it")

@@ -15,7 +15,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Any, Callable, Mapping
 
-ROLES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+ROLES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "entry")
 
 
 @dataclass(frozen=True)
@@ -135,3 +135,4 @@ def _load_builtin() -> None:
     from . import parts  # noqa: F401  (registers part kinds)
     from .models import qwen3  # noqa: F401  (registers Qwen3ForCausalLM; its presets come first)
     from .models import deginex  # noqa: F401  (registers Deginex)
+    from .models import zisedra  # noqa: F401  (registers Zisedra)

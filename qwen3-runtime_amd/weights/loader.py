@@ -50,13 +50,18 @@ class WeightError(RuntimeError):
         super().__init__("\n".join(lines))
 
 
+def _fits(got: tuple, want: tuple) -> bool:
+    """Whether a stored shape is the declared one; a declared size of -1 takes any."""
+    return len(got) == len(want) and all(w == -1 or w == g for g, w in zip(got, want))
+
+
 def check_source(source, decls: Sequence[TensorDecl], ignorable: Sequence[str] = (), where: str = "") -> None:
     wanted = {d.file_name: tuple(d.shape) for d in decls}
     missing = [n for n in wanted if not source.has(n)]
     wrong = [
         (n, source.shape(n), shape)
         for n, shape in wanted.items()
-        if source.has(n) and tuple(source.shape(n)) != shape
+        if source.has(n) and not _fits(tuple(source.shape(n)), shape)
     ]
     wrong_dtype = []
     for d in decls:

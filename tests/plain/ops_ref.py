@@ -21,9 +21,11 @@ def embed(ids, table):
     return table[ids.long()].to(torch.float32)
 
 
-def add_rmsnorm(residual, delta, weight, eps, out_dtype, rows=None, compute=torch.float32):
+def add_rmsnorm(residual, delta, weight, eps, out_dtype, rows=None, compute=torch.float32, delta_scale=1.0):
     if delta is not None and delta.dim() == 3:
         delta = delta.to(residual.dtype).sum(0)
+    if delta is not None and delta_scale != 1.0:
+        delta = delta.to(residual.dtype) * delta_scale
     if delta is not None:
         if rows is None:
             residual += delta.to(residual.dtype)
@@ -185,17 +187,37 @@ def mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows=None, com
     return y.to(out_dtype)
 
 
-def route_top(x, router, router_bias, top):
+def route_top(x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None):
     """float32 logits x W^T + b; the ``top`` largest per token (ties: the lower index first) and
-    the softmax over those alone. Returns (int32 [T, top], float32 [T, top])."""
+    the softmax over those alone. Returns (int32 [T, top], float32 [T, top]). With sigmoid scoring
+    the scores are the weights; with groups only the best ``keep`` groups' experts can be chosen."""
     logits = x.to(torch.float32) @ router.to(torch.float32).T
     if router_bias is not None:
         logits = logits + router_bias.to(torch.float32)
-    best, index = torch.topk(logits, top, dim=-1)
-    return index.to(torch.int32), torch.softmax(best, dim=-1)
+    values = torch.sigmoid(logits) if scoring == "sigmoid" else logits
+    pick = values
+    if groups > 1 and keep is not None and keep < groups:
+        t, e = values.shape
+        per = e // groups
+        g = values.view(t, groups, per)
+        gscore = torch.topk(g, min(2, per), dim=-1).values.sum(-1)
+        stay = torch.zeros(t, groups, dtype=torch.bool, device=x.device)
+        stay.scatter_(1, torch.topk(gscore, keep, dim=-1).indices, True)
+        pick = torch.where(stay[:, :, None].expand(t, groups, per).reshape(t, e), values,
+                           torch.full_like(values, float("-inf")))
+    best, index = torch.topk(pick, top, dim=-1)
+    return index.to(torch.int32), best if scoring == "sigmoid" else torch.softmax(best, dim=-1)
 
 
-def moe_swiglu(x, gate_up, down, index, weight, compute=torch.float32):
+def gated(g, u, activation="swiglu", limit=0.0):
+    if activation == "clamped":
+        g = torch.clamp(g, max=limit)
+        u = torch.clamp(u, min=-limit, max=limit)
+        return g * torch.sigmoid(1.702 * g) * (u + 1)
+    return g * torch.sigmoid(g) * u
+
+
+def moe_swiglu(x, gate_up, down, index, weight, compute=torch.float32, activation="swiglu", limit=0.0):
     """x [T, H]; gate_up [E, 2I, H]; down [E, H, I]; index/weight [T, top] -> [T, H] (float32)."""
     t, h = x.shape
     inter = gate_up.shape[1] // 2
@@ -205,7 +227,7 @@ def moe_swiglu(x, gate_up, down, index, weight, compute=torch.float32):
         for e in index[:, j].unique().tolist():
             sel = (index[:, j] == e).nonzero()[:, 0]
             gu = (xc[sel] @ gate_up[e].to(compute).T).to(x.dtype).to(compute)
-            act = (gu[:, :inter] * torch.sigmoid(gu[:, :inter]) * gu[:, inter:]).to(x.dtype).to(compute)
+            act = gated(gu[:, :inter], gu[:, inter:], activation, limit).to(x.dtype).to(compute)
             out[sel] += weight[sel, j, None] * (act @ down[e].to(compute).T).to(torch.float32)
     return out
 
@@ -214,6 +236,94 @@ def swiglu(gate_up, compute=torch.float32):
     i = gate_up.shape[-1] // 2
     g, u = gate_up[..., :i].to(compute), gate_up[..., i:].to(compute)
     return (g * torch.sigmoid(g) * u).to(gate_up.dtype)
+
+
+def planes_sum(y):
+    return y.to(torch.float32).sum(0) if y.dim() == 3 else y.to(torch.float32)
+
+
+def norm_mean(ya, wa, yb, wb, eps):
+    def normed(y, w):
+        y = planes_sum(y)
+        return y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps) * w
+    return 0.5 * (normed(ya, wa) + normed(yb, wb))
+
+
+def bias_rotate_pairs(x, bias, positions, freq, rot_heads, head_dim):
+    t, w = x.shape
+    y = x.to(torch.float32)
+    if bias is not None:
+        y = y + bias
+    if freq is not None and freq.numel():
+        n = freq.numel()
+        heads = y[:, : rot_heads * head_dim].reshape(t, rot_heads, head_dim).clone()
+        ang = positions.to(torch.float32)[:, None] * freq[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        a, b = heads[..., 0: 2 * n: 2].clone(), heads[..., 1: 2 * n: 2].clone()
+        heads[..., 0: 2 * n: 2] = a * cos - b * sin
+        heads[..., 1: 2 * n: 2] = b * cos + a * sin
+        y = torch.cat([heads.reshape(t, -1), y[:, rot_heads * head_dim:]], dim=1)
+    x.copy_(y.to(x.dtype))
+    return x
+
+
+def delta_conv(y, channels, taps, tail, cu_q, slots, segments, unit_eps):
+    """Causal convolution + silu + unit vectors per head, span by span; ``tail`` updated in place."""
+    k = taps.shape[1]
+    out = torch.empty((y.shape[0], channels), dtype=torch.float32, device=y.device)
+    for s in range(len(cu_q) - 1):
+        a, b = int(cu_q[s]), int(cu_q[s + 1])
+        slot = int(slots[s])
+        x = y[a:b, :channels].to(torch.float32)
+        full = torch.cat([tail[slot, :, : k - 1].T, x], dim=0) if k > 1 else x
+        acc = torch.zeros_like(x)
+        for j in range(k):
+            acc = acc + full[j: j + (b - a)] * taps[:, j]
+        out[a:b] = acc * torch.sigmoid(acc)
+        if k > 1:
+            tail[slot, :, : k - 1] = full[full.shape[0] - (k - 1):].T
+    first = 0
+    for heads, width, mode in segments:
+        if mode:
+            seg = out[:, first: first + heads * width].view(-1, heads, width)
+            seg = seg / torch.sqrt(seg.pow(2).sum(-1, keepdim=True) + unit_eps)
+            if mode == 2:
+                seg = seg * width ** -0.5
+            out[:, first: first + heads * width] = seg.reshape(-1, heads * width)
+        first += heads * width
+    return out
+
+
+def delta_rule(qkv, beta, a_logits, a_log, dt_bias, state, cu_q, slots, heads, kv_heads, dim, vdim, per_channel):
+    t = qkv.shape[0]
+    q = qkv[:, : kv_heads * dim].view(t, kv_heads, dim)
+    k = qkv[:, kv_heads * dim: 2 * kv_heads * dim].view(t, kv_heads, dim)
+    v = qkv[:, 2 * kv_heads * dim:].view(t, heads, vdim)
+    b = torch.sigmoid(beta.to(torch.float32))
+    sp = torch.nn.functional.softplus(a_logits.to(torch.float32) + dt_bias)
+    rate = torch.exp(a_log)
+    g = torch.exp(-rate[None, :, None] * sp.view(t, heads, dim)) if per_channel else torch.exp(-rate[None, :] * sp)
+    out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qkv.device)
+    group = heads // kv_heads
+    for s in range(len(cu_q) - 1):
+        slot = int(slots[s])
+        for h in range(heads):
+            st = state[slot, h].T.clone()  # [dim, vdim]
+            for i in range(int(cu_q[s]), int(cu_q[s + 1])):
+                st = st * (g[i, h][:, None] if per_channel else g[i, h])
+                u = b[i, h] * (v[i, h] - st.T @ k[i, h // group])
+                st = st + torch.outer(k[i, h // group], u)
+                out[i, h] = st.T @ q[i, h // group]
+            state[slot, h] = st.T
+    return out
+
+
+def delta_out(o, weight, gate, eps, gate_kind, out_dtype):
+    t, heads, vdim = o.shape
+    z = gate.to(torch.float32).view(t, heads, vdim)
+    act = z * torch.sigmoid(z) if gate_kind == "silu" else torch.sigmoid(z)
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * weight * act
+    return y.reshape(t, heads * vdim).to(out_dtype)
 
 
 def argmax(logits):
@@ -229,8 +339,36 @@ class TorchOps:
     def embed(self, ids, table):
         return embed(ids, table)
 
-    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
-        return add_rmsnorm(residual, delta, weight, eps, out_dtype, rows, self.compute)
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, delta_scale=1.0):
+        return add_rmsnorm(residual, delta, weight, eps, out_dtype, rows, self.compute, delta_scale)
+
+    def norm_mean(self, ya, wa, yb, wb, eps):
+        return norm_mean(ya, wa, yb, wb, eps)
+
+    def add_concat(self, residual, delta, delta_scale, origin, out_dtype):
+        x = residual if delta is None else residual + delta_scale * planes_sum(delta)
+        return torch.cat([x, origin], dim=1).to(out_dtype)
+
+    def accumulate(self, acc, y):
+        acc += planes_sum(y)
+        return acc
+
+    def gated_act(self, gate_up, activation="swiglu", limit=0.0):
+        i = gate_up.shape[-1] // 2
+        return gated(gate_up[..., :i].to(self.compute), gate_up[..., i:].to(self.compute), activation, limit).to(gate_up.dtype)
+
+    def bias_rotate_pairs(self, x, bias, positions, freq, rot_heads, head_dim):
+        return bias_rotate_pairs(x, bias, positions, freq, rot_heads, head_dim)
+
+    def delta_conv(self, ctx, y, channels, taps, tail, segments, unit_eps):
+        return delta_conv(y, channels, taps, tail, ctx.cu_q, ctx.state_slots, segments, unit_eps)
+
+    def delta_rule(self, ctx, qkv, beta, a_logits, a_log, dt_bias, state, heads, kv_heads, dim, vdim, per_channel):
+        return delta_rule(qkv, beta, a_logits, a_log, dt_bias, state, ctx.cu_q, ctx.state_slots, heads, kv_heads,
+                          dim, vdim, per_channel)
+
+    def delta_out(self, o, weight, gate, eps, gate_kind, out_dtype):
+        return delta_out(o, weight, gate, eps, gate_kind, out_dtype)
 
     def linear(self, x, w, out_f32=False):
         return linear(x, w, out_f32, self.compute)
@@ -250,11 +388,11 @@ class TorchOps:
     def mix_norm(self, streams, update, read, weight, bias, eps, out_dtype, rows=None):
         return mix_norm(streams, update, read, weight, bias, eps, out_dtype, rows, self.compute)
 
-    def route_top(self, x, router, router_bias, top):
-        return route_top(x, router, router_bias, top)
+    def route_top(self, x, router, router_bias, top, scoring="softmax_top", groups=1, keep=None):
+        return route_top(x, router, router_bias, top, scoring, groups, keep)
 
-    def moe_swiglu(self, x, gate_up, down, index, weight):
-        return moe_swiglu(x, gate_up, down, index, weight, self.compute)
+    def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0):
+        return moe_swiglu(x, gate_up, down, index, weight, self.compute, activation, limit)
 
     def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache, **more):
         return False  # no one-kernel form of a decode step's attention here: the steps above, in order
@@ -278,8 +416,8 @@ class TorchOps:
     def swiglu(self, gate_up):
         return swiglu(gate_up, self.compute)
 
-    def gated_linear(self, x, w_gate_up):
-        return swiglu(linear(x, w_gate_up, False, self.compute), self.compute)
+    def gated_linear(self, x, w_gate_up, activation="swiglu", limit=0.0):
+        return self.gated_act(linear(x, w_gate_up, False, self.compute), activation, limit)
 
     def argmax(self, logits):
         return argmax(logits)
