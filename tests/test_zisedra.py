@@ -440,9 +440,29 @@ def config_c():
                 {"type": "delta", "mixer": delta(1, 1, 64, 128, 2), "mlp": None}]}, 16
 
 
+def every_expert(make):
+    """The same model with a router that has no choice to make (every expert of every group is taken,
+    weighted by its score): for runs in bfloat16, where a choice between two experts whose scores
+    lie within rounding of each other may fall the other way, which moves that position's logits by
+    a large part of their spread, and later positions' through the recurrent state. The choice
+    itself is held to the plain one in float32 here, and in both types in the router's own test."""
+    def made():
+        raw, page = make()
+        for layer in raw["layers"]:
+            if layer["mlp"]:
+                router = layer["mlp"]["router"]
+                router["top"], router["groups"]["keep"] = router["experts"], router["groups"]["count"]
+        return raw, page
+    return made
+
+
 CONFIGS = {"a": config_a, "b": config_b, "c": config_c}
-# share of positions at which a router may choose differently in bfloat16
-FLIPS = {"a": 0.12, "b": 0.06, "c": 0.08}
+CONFIGS.update({name + "_every": every_expert(make) for name, make in list(CONFIGS.items())})
+# bfloat16: the bound on the largest error of a position's logits, in units of their deviation. The
+# error has a long tail: over six seeds of "c" its median per position was 0.02 and the largest
+# 0.13 to 0.46, at scattered positions; "a" (eight layer runs of width 96, a gain above one at
+# every entry of its loop) measured 0.37, "b" 0.11. float32 showed no error in any of them.
+NOISE = {"a": 0.6, "b": 0.3, "c": 0.6}
 LENGTHS = {"a": [1, 7, 45, 130], "b": [3, 17, 50, 64, 101], "c": [2, 16, 17, 120]}
 _folders: dict = {}
 
@@ -451,7 +471,9 @@ _folders: dict = {}
 def folder(tmp_path_factory):
     from qwen3_runtime_amd.weights import write_model_folder
 
-    def get(name):
+    def get(name, dtype="float32"):
+        if dtype == "bfloat16":
+            name += "_every"
         if name not in _folders:
             raw, _ = CONFIGS[name]()
             _folders[name] = write_model_folder(tmp_path_factory.mktemp("zisedra_" + name), raw, seed=71 + len(_folders),
@@ -481,12 +503,10 @@ def plain_logits(folder, requests):
     return out
 
 
-def check(got, want, dtype, flips=0.03):
+def check(got, want, dtype, noise=0.2):
     """float32: to rounding of float32 sums, everywhere. bfloat16: as noise relative to the logits'
-    own spread; a router is a hard choice, and where two experts' scores lie within rounding of
-    each other bfloat16 may take the other one, which moves that position's logits (and, through
-    the recurrent state, later ones a little). So up to ``flips`` of the positions may lie over the
-    bound; a wrong window, state or portion shows in float32, where no position may."""
+    own spread, no position over ``noise`` and their root mean square under a quarter of it; a wrong
+    window, state or portion shows in float32, where the bound is rounding."""
     if dtype == "float32":
         traces.compare(got, want, atol=2e-4, rtol=2e-4)
         return
@@ -496,15 +516,15 @@ def check(got, want, dtype, flips=0.03):
     err = torch.stack([got[k].double() for k in keys]) - w
     std = float(w.std())
     per_pos = err.abs().amax(dim=1)
-    good = per_pos < 0.12 * std
-    assert int((~good).sum()) <= flips * len(keys), \
+    good = per_pos < noise * std
+    assert bool(good.all()), \
         f"{int((~good).sum())} of {len(keys)} positions over the bound, the first {keys[int((~good).nonzero()[0])]}"
-    rms = float(err[good].pow(2).mean().sqrt())
-    assert rms < 0.03 * std, f"rms error {rms:.4f} against a logit deviation of {std:.3f}"
+    rms = float(err.pow(2).mean().sqrt())
+    assert rms < 0.25 * noise * std, f"rms error {rms:.4f} against a logit deviation of {std:.3f}"
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", list(CONFIGS))
+@pytest.mark.parametrize("name", ["a", "b", "c"])
 @pytest.mark.parametrize("cut", ["whole", "tail_one_by_one", "portions", "mixed"])
 def test_cuttings_match_plain(folder, backend, name, cut):
     """Whole prompts; the last tokens one by one (across window edges); portions down to two tokens;
@@ -513,9 +533,9 @@ def test_cuttings_match_plain(folder, backend, name, cut):
     raw, page = CONFIGS[name]()
     reqs = traces.make_requests(raw["vocab"], LENGTHS[name] + ([30, 9] if cut == "mixed" else []), seed=5)
     steps = getattr(traces, cut)(reqs)
-    loaded = load(folder(name), page, traces.peak_tokens(steps, unit=page) // page, backend)
+    loaded = load(folder(name, backend[1]), page, traces.peak_tokens(steps, unit=page) // page, backend)
     got = traces.replay(loaded, steps, poison_freed=True)
-    check(got, plain_logits(folder(name), reqs), backend[1], flips=FLIPS[name])
+    check(got, plain_logits(folder(name, backend[1]), reqs), backend[1], NOISE[name])
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
@@ -525,9 +545,9 @@ def test_long_decoding_in_a_pool_of_one_window(folder, backend):
     raw, page = config_b()
     reqs = traces.make_requests(raw["vocab"], [300], seed=8)
     steps = traces.tail_one_by_one(reqs, tail=290)
-    loaded = load(folder("b"), page, 4, backend)
+    loaded = load(folder("b", backend[1]), page, 4, backend)
     got = traces.replay(loaded, steps, poison_freed=True)
-    check(got, plain_logits(folder("b"), reqs), backend[1], flips=FLIPS["b"])
+    check(got, plain_logits(folder("b", backend[1]), reqs), backend[1], NOISE["b"])
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
@@ -537,13 +557,13 @@ def test_batch_mates_do_not_change_a_request(folder, backend):
     reqs = traces.make_requests(raw["vocab"], [9, 60, 121, 33], seed=2)
     together = [{"step": 0, "entries": [{"id": r, "tokens": t, "want": list(range(len(t)))} for r, t in reqs.items()],
                  "end": list(reqs)}]
-    loaded = load(folder("a"), page, 32, backend)
+    loaded = load(folder("a", backend[1]), page, 32, backend)
     both = traces.replay(loaded, together)
     alone = traces.replay(loaded, traces.whole(reqs))
     if backend[1] == "float32":
         traces.compare(both, alone, atol=2e-5, rtol=2e-5)
     else:
-        check(both, alone, "bfloat16", flips=FLIPS["a"])
+        check(both, alone, "bfloat16", NOISE["a"])
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
@@ -574,18 +594,17 @@ def test_greedy_generation_through_the_entry_point(folder, name, dtype, graphs):
     from qwen3_runtime_amd.llm import LLM
 
     raw, page = CONFIGS[name]()
-    llm = LLM(str(folder(name)), dtype=dtype, block_size=page, num_kv_blocks=64, max_num_seqs=3,
+    llm = LLM(str(folder(name, dtype)), dtype=dtype, block_size=page, num_kv_blocks=64, max_num_seqs=3,
               max_num_batched_tokens=48, cuda_graph=graphs)
     prompts = list(traces.make_requests(raw["vocab"], [5, 61, 20, 90], seed=4).values())
     outs = llm.generate(prompts, max_tokens=40)
-    cfg, w = P.load(folder(name))
+    cfg, w = P.load(folder(name, dtype))
     for prompt, tokens in zip(prompts, outs):
         assert len(tokens) == 40
         logits = P.forward(cfg, w, list(prompt) + list(tokens))[len(prompt) - 1: -1]
         below = logits.max(-1).values - logits[range(40), list(tokens)]
-        bound = 1e-3 if dtype == "float32" else 0.12 * float(logits.std())
-        allowed = 0 if dtype == "float32" else int(FLIPS[name] * 40)
-        assert int((below >= bound).sum()) <= allowed, (float(below.max()), int(below.argmax()))
+        bound = 1e-3 if dtype == "float32" else 2 * NOISE[name] * float(logits.std())
+        assert int((below >= bound).sum()) == 0, (float(below.max()), int(below.argmax()))
 
 
 # ------------------------------------------------------------------ configuration and plan
