@@ -18,21 +18,45 @@ __device__ __forceinline__ float planes_at(const Planes& y, size_t i) {
   return v;
 }
 
-// out[t] = (1/2) (a[t] / rms(a[t]) * wa + b[t] / rms(b[t]) * wb), rms with eps inside the root
-__global__ __launch_bounds__(256) void norm_mean_kernel(Planes ya, Planes yb, const float* __restrict__ wa,
-                                                        const float* __restrict__ wb, float* __restrict__ out,
-                                                        int hidden, float eps) {
+// out[t] = (1/2) (a[t] / rms(a[t]) * wa + b[t] / rms(b[t]) * wb), rms with eps inside the root.
+// One block of 1,024 threads per token; a thread keeps its elements of both rows in registers
+// (rows up to 4,096 wide; wider rows are read a second time), and asks for all of them, and for
+// the weights, before the first use: a token costs one round of memory latency.
+#define NM_KEEP 4
+__global__ __launch_bounds__(1024) void norm_mean_kernel(Planes ya, Planes yb, const float* __restrict__ wa,
+                                                         const float* __restrict__ wb, float* __restrict__ out,
+                                                         int hidden, float eps) {
   __shared__ float red[32];
   const size_t row = (size_t)blockIdx.x * hidden;
+  float va[NM_KEEP], vb[NM_KEEP], ua[NM_KEEP], ub[NM_KEEP];
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = min((int)threadIdx.x + 1024 * j, hidden - 1);  // beyond the row: its last element, dropped below
+    va[j] = planes_at(ya, row + i);
+    vb[j] = planes_at(yb, row + i);
+    ua[j] = wa[i];
+    ub[j] = wb[i];
+  }
   float sa = 0.f, sb = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += 256) {
-    const float va = planes_at(ya, row + i), vb = planes_at(yb, row + i);
-    sa += va * va;
-    sb += vb * vb;
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j)
+    if ((int)threadIdx.x + 1024 * j < hidden) {
+      sa += va[j] * va[j];
+      sb += vb[j] * vb[j];
+    }
+  for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024) {
+    const float x = planes_at(ya, row + i), y = planes_at(yb, row + i);
+    sa += x * x;
+    sb += y * y;
   }
   const float ia = 1.0f / sqrtf(block_sum(sa, red) / (float)hidden + eps);
   const float ib = 1.0f / sqrtf(block_sum(sb, red) / (float)hidden + eps);
-  for (int i = threadIdx.x; i < hidden; i += 256)
+#pragma unroll
+  for (int j = 0; j < NM_KEEP; ++j) {
+    const int i = threadIdx.x + 1024 * j;
+    if (i < hidden) out[row + i] = 0.5f * (va[j] * ia * ua[j] + vb[j] * ib * ub[j]);
+  }
+  for (int i = threadIdx.x + 1024 * NM_KEEP; i < hidden; i += 1024)
     out[row + i] = 0.5f * (planes_at(ya, row + i) * ia * wa[i] + planes_at(yb, row + i) * ib * wb[i]);
 }
 
@@ -44,7 +68,7 @@ extern "C" int qrt_norm_mean(const void* a, int a_code, int a_planes, const void
             "norm_mean: planes are float32");
   if (num_tokens == 0) return 0;
   const long stride = (long)num_tokens * hidden;
-  norm_mean_kernel<<<dim3(num_tokens), 256, 0, stream>>>(Planes{a, a_code, a_planes, stride}, Planes{b, b_code, b_planes, stride},
+  norm_mean_kernel<<<dim3(num_tokens), 1024, 0, stream>>>(Planes{a, a_code, a_planes, stride}, Planes{b, b_code, b_planes, stride},
                                                          wa, wb, out, hidden, eps);
   QRT_LAUNCH_CHECK("norm_mean");
   return 0;

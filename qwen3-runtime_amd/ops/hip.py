@@ -388,7 +388,7 @@ class HipOps:
         a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
         a.state_slots = _need(ctx.state_slots, "state_slots", torch.int32, (ctx.num_seqs,)).data_ptr()
         a.heads, a.kv_heads, a.dim, a.vdim, a.per_channel = heads, kv_heads, dim, vdim, int(bool(per_channel))
-        self._check(self.lib, self.lib.qrt_delta_rule(byref(a), c_int(t), c_int(ctx.num_seqs), _stream()))
+        self._check(self.lib, self.lib.qrt_delta_rule(byref(a), c_int(t), c_int(ctx.num_seqs), c_int(ctx.max_q_len), _stream()))
         return out
 
     def delta_out(self, o, weight, gate, eps, gate_kind, out_dtype):
