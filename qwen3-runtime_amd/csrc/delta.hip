@@ -35,6 +35,9 @@ struct ConvArgs {
   int seg_first[4], seg_heads[4], seg_width[4], seg_mode[4];
   int total_heads;
   float unit_eps;
+  // every span is one token (a decode step): the wave that reads a channel's tail also moves it on,
+  // and no second kernel runs
+  int fuse_tail;
 };
 
 template <typename T>
@@ -51,7 +54,7 @@ __global__ __launch_bounds__(256) void conv_unit_kernel(ConvArgs a) {
   const int s = a.seq_of_token[t];
   const int i = t - a.cu_q[s];            // place within the span
   const int K = a.num_taps;
-  const float* tail = a.tail + (size_t)a.state_slots[s] * a.channels * (K - 1);
+  float* tail = (float*)a.tail + (size_t)a.state_slots[s] * a.channels * (K - 1);
   const T* x = (const T*)a.x;
   float ss = 0.f;
   float y[8];
@@ -66,6 +69,7 @@ __global__ __launch_bounds__(256) void conv_unit_kernel(ConvArgs a) {
         const float in = back <= i ? to_f32<T>(x[(size_t)(t - back) * a.x_stride + c])
                                    : tail[(size_t)c * (K - 1) + (i + j)];
         acc = fmaf(a.taps[(size_t)c * K + j], in, acc);
+        if (a.fuse_tail && j >= 1) tail[(size_t)c * (K - 1) + (j - 1)] = in;  // i is 0: the inputs were tail[0..K-2], x
       }
       y[r] = acc / (1.0f + expf(-acc));
       ss += y[r] * y[r];
@@ -80,6 +84,99 @@ __global__ __launch_bounds__(256) void conv_unit_kernel(ConvArgs a) {
 #pragma unroll
   for (int r = 0; r < 8; ++r)
     if (lane + 64 * r < width) a.out[(size_t)t * a.channels + c0 + lane + 64 * r] = y[r] * mul;
+}
+
+// The same for steps of many tokens, K <= 4 taps and heads of at most 128 channels: a wave takes
+// eight consecutive tokens of one head, loads the 8 + K - 1 rows of inputs they read once (a
+// window in registers; the taps once), and computes the eight outputs from it. A token near the
+// start of its span reads the slot's tail instead of the rows before it, which belong to another
+// sequence of the batch.
+#define CONV_TILE 8
+template <typename T, int K>
+__global__ __launch_bounds__(256) void conv_unit_tile_kernel(ConvArgs a) {
+  const int lane = threadIdx.x & 63;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int tiles = (a.num_tokens + CONV_TILE - 1) / CONV_TILE;
+  if (item >= (long)tiles * a.total_heads) return;
+  const int tile = (int)(item / a.total_heads);
+  int h = (int)(item - (long)tile * a.total_heads);
+  int seg = 0;
+  while (seg + 1 < a.nseg && h >= a.seg_heads[seg]) { h -= a.seg_heads[seg]; ++seg; }
+  const int width = a.seg_width[seg], mode = a.seg_mode[seg];
+  const int c0 = a.seg_first[seg] + h * width;
+  const int t0 = tile * CONV_TILE, nt = min(CONV_TILE, a.num_tokens - t0);
+  const T* x = (const T*)a.x;
+  float w[2][K], xw[2][CONV_TILE + K - 1], y[2][CONV_TILE];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const bool on = lane + 64 * r < width;
+    const int c = c0 + (on ? lane + 64 * r : 0);
+#pragma unroll
+    for (int j = 0; j < K; ++j) w[r][j] = a.taps[(size_t)c * K + j];
+#pragma unroll
+    for (int j = 0; j < CONV_TILE + K - 1; ++j) {
+      const int row = t0 - (K - 1) + j;
+      const int at = min(max(row, 0), a.num_tokens - 1);
+      const float v = to_f32<T>(x[(size_t)at * a.x_stride + c]);
+      xw[r][j] = (on && row >= 0 && row < a.num_tokens) ? v : 0.f;
+    }
+  }
+  float ss[CONV_TILE];
+#pragma unroll
+  for (int tt = 0; tt < CONV_TILE; ++tt) {
+    ss[tt] = 0.f;
+    const int t = min(t0 + tt, a.num_tokens - 1);
+    const int s = a.seq_of_token[t];
+    const int i = t - a.cu_q[s];
+    const float* tail = a.tail + (size_t)a.state_slots[s] * a.channels * (K - 1);
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        float in = xw[r][tt + j];
+        if (K - 1 - j > i) in = (lane + 64 * r < width) ? tail[(size_t)(c0 + lane + 64 * r) * (K - 1) + (i + j)] : 0.f;
+        acc = fmaf(w[r][j], in, acc);
+      }
+      y[r][tt] = acc / (1.0f + __expf(-acc));
+      ss[tt] += y[r][tt] * y[r][tt];
+    }
+  }
+  if (mode) {
+#pragma unroll
+    for (int tt = 0; tt < CONV_TILE; ++tt) {
+      const float total = wave_sum(ss[tt]);
+      ss[tt] = 1.0f / sqrtf(total + a.unit_eps);
+      if (mode == 2) ss[tt] *= 1.0f / sqrtf((float)width);
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < CONV_TILE; ++tt) {
+    if (tt < nt) {
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+        if (lane + 64 * r < width)
+          a.out[(size_t)(t0 + tt) * a.channels + c0 + lane + 64 * r] = mode ? y[r][tt] * ss[tt] : y[r][tt];
+    }
+  }
+}
+
+template <typename T>
+static void conv_launch(const ConvArgs& a, bool tiled, hipStream_t stream) {
+  if (tiled) {
+    const long items = (long)((a.num_tokens + CONV_TILE - 1) / CONV_TILE) * a.total_heads;
+    dim3 grid((unsigned)((items + 3) / 4)), block(256);
+    switch (a.num_taps) {
+      case 1: conv_unit_tile_kernel<T, 1><<<grid, block, 0, stream>>>(a); break;
+      case 2: conv_unit_tile_kernel<T, 2><<<grid, block, 0, stream>>>(a); break;
+      case 3: conv_unit_tile_kernel<T, 3><<<grid, block, 0, stream>>>(a); break;
+      default: conv_unit_tile_kernel<T, 4><<<grid, block, 0, stream>>>(a); break;
+    }
+  } else {
+    const long items = (long)a.num_tokens * a.total_heads;
+    dim3 grid((unsigned)((items + 3) / 4)), block(256);
+    conv_unit_kernel<T><<<grid, block, 0, stream>>>(a);
+  }
 }
 
 // After the convolution has read them: the tail of every (sequence, channel) becomes the last
@@ -101,8 +198,10 @@ __global__ void conv_tail_kernel(const T* __restrict__ x, long x_stride, float* 
   for (int r = 0; r < K - 1; ++r) tail[r] = keep[r];
 }
 
-extern "C" int qrt_delta_conv(const ConvArgs* args, int dtype, int num_seqs, int num_slots, hipStream_t stream) {
+extern "C" int qrt_delta_conv(const ConvArgs* args, int dtype, int num_seqs, int num_slots, int max_span,
+                              hipStream_t stream) {
   ConvArgs a = *args;
+  a.fuse_tail = max_span == 1 && a.num_tokens == num_seqs;
   QRT_CHECK(a.num_tokens >= 0 && a.channels > 0 && a.nseg >= 1 && a.nseg <= 4, "delta_conv: bad sizes");
   QRT_CHECK(a.num_taps >= 1 && a.num_taps <= DELTA_MAX_TAPS, "delta_conv: %d taps (1 to %d)", a.num_taps, DELTA_MAX_TAPS);
   QRT_CHECK(a.x_stride >= a.channels && num_seqs >= 0 && num_slots > 0, "delta_conv: row stride %ld under %d channels", a.x_stride, a.channels);
@@ -116,17 +215,17 @@ extern "C" int qrt_delta_conv(const ConvArgs* args, int dtype, int num_seqs, int
   }
   QRT_CHECK(covered == a.channels, "delta_conv: segments cover %d of %d channels", covered, a.channels);
   if (a.num_tokens == 0) return 0;
-  const long items = (long)a.num_tokens * a.total_heads;
-  dim3 grid((unsigned)((items + 3) / 4)), block(256);
+  bool tiled = a.num_tokens >= 64 && a.num_taps <= 4 && !a.fuse_tail;
+  for (int g = 0; g < a.nseg; ++g) tiled = tiled && a.seg_width[g] <= 128;
   dim3 tgrid((a.channels + 255) / 256, num_seqs);
   if (dtype == QRT_F32) {
-    conv_unit_kernel<float><<<grid, block, 0, stream>>>(a);
-    if (a.num_taps > 1)
+    conv_launch<float>(a, tiled, stream);
+    if (a.num_taps > 1 && !a.fuse_tail)
       conv_tail_kernel<float><<<tgrid, 256, 0, stream>>>((const float*)a.x, a.x_stride, (float*)a.tail, a.cu_q,
                                                         a.state_slots, a.channels, a.num_taps);
   } else if (dtype == QRT_BF16) {
-    conv_unit_kernel<bf16_t><<<grid, block, 0, stream>>>(a);
-    if (a.num_taps > 1)
+    conv_launch<bf16_t>(a, tiled, stream);
+    if (a.num_taps > 1 && !a.fuse_tail)
       conv_tail_kernel<bf16_t><<<tgrid, 256, 0, stream>>>((const bf16_t*)a.x, a.x_stride, (float*)a.tail, a.cu_q,
                                                          a.state_slots, a.channels, a.num_taps);
   } else return qrt_fail("delta_conv: unknown dtype %d", dtype);

@@ -129,3 +129,4 @@ for _name, _cfg in PRESETS.items():
 # the sizes of the 4B dense preset, for measurements beside it
 register_preset("deginex_4b", sized(2560, 36, 32, 8, 128, 9728, 151936).to_dict(), 16)
 register_preset("deginex_4b_moe", sized(2560, 36, 32, 8, 128, 9728, 151936, experts=16, top=2, expert_ff=1536).to_dict(), 16)
+register_preset("deginex_8b_moe", sized(4096, 36, 32, 8, 128, 12288, 151936, experts=16, top=2, expert_ff=2048).to_dict(), 16)

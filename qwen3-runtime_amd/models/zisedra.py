@@ -147,5 +147,8 @@ def sized(width: int, layers: int, heads: int, kv_heads: int, dim: int, vocab: i
 register_architecture(ZisedraConfig.architecture, ZisedraConfig.from_dict, plan_zisedra)
 for _name, _cfg in PRESETS.items():
     register_preset(_name, _cfg.to_dict(), PRESET_PAGE_SIZE.get(_name, 16))
-# the sizes of the 4B dense preset's layers with a mixture like `deginex_4b_moe`'s, for measurements beside it
+# layers of the sizes of the 4B and 8B dense presets, and of a smaller width, with a mixture like
+# `deginex_4b_moe`'s in every layer, for measurements beside it
 register_preset("zisedra_4b", sized(2560, 36, 32, 8, 128, 151936, expert_ff=1536, shared_ff=1536).to_dict(), 16)
+register_preset("zisedra_8b", sized(4096, 36, 32, 8, 128, 151936, expert_ff=2048, shared_ff=2048).to_dict(), 16)
+register_preset("zisedra_2b", sized(2048, 28, 16, 4, 128, 151936, expert_ff=1024, shared_ff=1024).to_dict(), 16)

@@ -90,7 +90,7 @@ class _ConvArgs(Structure):
         ("cu_q", c_void_p), ("seq_of_token", c_void_p), ("state_slots", c_void_p), ("out", c_void_p),
         ("num_tokens", c_int), ("channels", c_int), ("num_taps", c_int), ("nseg", c_int),
         ("seg_first", c_int * 4), ("seg_heads", c_int * 4), ("seg_width", c_int * 4), ("seg_mode", c_int * 4),
-        ("total_heads", c_int), ("unit_eps", c_float),
+        ("total_heads", c_int), ("unit_eps", c_float), ("fuse_tail", c_int),
     ]
 
 
@@ -360,7 +360,8 @@ class HipOps:
             first += heads * width
         if first != channels:
             raise OpsError(f"delta_conv: segments cover {first} of {channels} channels")
-        self._check(self.lib, self.lib.qrt_delta_conv(byref(a), _CODE[y.dtype], c_int(ctx.num_seqs), c_int(slots), _stream()))
+        self._check(self.lib, self.lib.qrt_delta_conv(byref(a), _CODE[y.dtype], c_int(ctx.num_seqs), c_int(slots),
+                                                      c_int(ctx.max_q_len), _stream()))
         return out
 
     def delta_rule(self, ctx, qkv, beta, a_logits, a_log, dt_bias, state, heads, kv_heads, dim, vdim, per_channel):
@@ -466,7 +467,7 @@ class HipOps:
                                                      c_int(groups if keep is None else keep), _stream()))
         return index, weight
 
-    def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0):
+    def moe_swiglu(self, x, gate_up, down, index, weight, activation="swiglu", limit=0.0, out=None):
         """``sum_j weight[t, j] * down[e] (silu(gate[e] x) * (up[e] x))`` with ``e = index[t, j]``;
         ``gate_up`` [E, 2I, H] (gate rows first), ``down`` [E, H, I]. float32 [T, H]."""
         t, h = x.shape
@@ -478,7 +479,10 @@ class HipOps:
         _need(down, "expert down", x.dtype, (n, h, inter))
         _need(index, "expert index", torch.int32, (t, top))
         _need(weight, "expert weight", torch.float32, (t, top))
-        out = torch.empty((t, h), dtype=torch.float32, device=x.device)
+        if out is None:
+            out = torch.empty((t, h), dtype=torch.float32, device=x.device)
+        else:  # the caller's own float32 rows (a plane of a sum that the next norm adds up)
+            _need(out, "experts' output", torch.float32, (t, h))
         if t == 0:
             return out
         pairs = t * top
@@ -684,6 +688,28 @@ class HipOps:
         _need(x, "x", torch.bfloat16)
         _need(w, "weight", torch.bfloat16, (n, k))
         out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+        self._check(self.lib, self.lib.qrt_gemm_bf16(
+            _ptr(x), _ptr(w), _ptr(out), F32, c_int(m), c_int(n), c_int(k), c_int(0),
+            c_int(kernel), c_int(parts), _stream()))
+        return out
+
+    def linear_planes_with_spare(self, x, w):
+        """``linear_for_residual(x, w)`` as float32 planes ``[P + 1, T, N]`` of which the last is left
+        for the caller to fill with one more addend of the same sum (so that the sum costs no
+        kernel of its own); None where the product does not run in the engine's own kernels."""
+        m, k = x.shape
+        n = w.shape[0]
+        if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and k % 64 == 0):
+            return None
+        kernel = self._own_kernel(m, n, k, "planes")
+        if kernel is None:
+            return None
+        parts = self.choose_k_parts(n, k, m, kernel == 1)
+        if parts == 1 and m > self.own_max_rows:  # above that many rows only products cut along K have a kernel
+            return None
+        _need(x, "x", torch.bfloat16)
+        _need(w, "weight", torch.bfloat16, (n, k))
+        out = torch.empty((parts + 1, m, n), dtype=torch.float32, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
             _ptr(x), _ptr(w), _ptr(out), F32, c_int(m), c_int(n), c_int(k), c_int(0),
             c_int(kernel), c_int(parts), _stream()))

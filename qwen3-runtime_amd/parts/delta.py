@@ -88,7 +88,7 @@ class GatedDeltaRule(Mixer):
         for n, rows in self._head_rows()[:3]:
             decls.append(TensorDecl(self._name(n) + ".conv", (rows, self.taps)))
         per = self.heads if self.decay == "head" else self.heads * self.dim
-        decls += [TensorDecl(self._name("A_log"), (self.heads,), init="norm"),
+        decls += [TensorDecl(self._name("A_log"), (self.heads,), init="log_rate"),
                   TensorDecl(self._name("dt_bias"), (per,)),
                   TensorDecl(self._name("norm"), (self.vdim,), init="norm"),
                   TensorDecl(self._name("o"), (h, self.heads * self.vdim))]

@@ -108,12 +108,18 @@ class RoutedSwiGLU(FeedForward):
         plain = self.scoring == "softmax_top" and self.groups == 1 and self.activation == "swiglu"
         if plain:
             index, weight = ops.route_top(x, self.router, self.router_bias, self.top)
-            out = ops.moe_swiglu(x, self.gate_up, self.down, index, weight)
-        else:
-            index, weight = ops.route_top(x, self.router, self.router_bias, self.top, scoring=self.scoring,
-                                          groups=self.groups, keep=self.keep)
-            out = ops.moe_swiglu(x, self.gate_up, self.down, index, weight, activation=self.activation, limit=self.limit)
-        if self.shared_size:
-            act = ops.gated_linear(x, self.shared_gate_up, activation=self.activation, limit=self.shared_limit)
-            out = ops.accumulate(out, ops.linear_for_residual(act, self.shared_down))
-        return out
+            return ops.moe_swiglu(x, self.gate_up, self.down, index, weight)
+        index, weight = ops.route_top(x, self.router, self.router_bias, self.top, scoring=self.scoring,
+                                      groups=self.groups, keep=self.keep)
+        more = {"activation": self.activation, "limit": self.limit}
+        if not self.shared_size:
+            return ops.moe_swiglu(x, self.gate_up, self.down, index, weight, **more)
+        act = ops.gated_linear(x, self.shared_gate_up, activation=self.activation, limit=self.shared_limit)
+        # few tokens: the shared expert's product leaves float32 planes with one to spare, the routed
+        # experts write theirs into it, and the norm that comes next adds them all up
+        planes = ops.linear_planes_with_spare(act, self.shared_down)
+        if planes is not None:
+            ops.moe_swiglu(x, self.gate_up, self.down, index, weight, out=planes[-1], **more)
+            return planes
+        out = ops.moe_swiglu(x, self.gate_up, self.down, index, weight, **more)
+        return ops.accumulate(out, ops.linear_for_residual(act, self.shared_down))

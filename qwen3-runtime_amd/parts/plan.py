@@ -34,7 +34,8 @@ class TensorDecl:
 
     ``init`` tells the random-weights mode how to draw it: ``"matrix"`` and
     ``"embedding"`` are zero-mean normal, ``"norm"`` is a scale around one, ``"mixing"``
-    a square matrix around the identity.
+    a square matrix around the identity, ``"log_rate"`` the logarithm of a decay rate (around -2:
+    a recurrent state that forgets over tens of tokens).
     ``storage`` is ``"float"`` (stored as bfloat16, float32 or float16) or ``"int"``
     (an integer table, held as int32; drawn as zeros in the random-weights mode unless
     ``init`` is ``"index:<n>"``, uniform in ``[0, n)``).

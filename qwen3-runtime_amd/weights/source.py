@@ -118,6 +118,8 @@ class RandomSource:
         x = torch.randn(decl.shape, generator=gen, dtype=torch.float32, device=device)
         if decl.init == "norm":
             x = 1.0 + self.norm_jitter * x
+        elif decl.init == "log_rate":
+            x = -2.0 + x
         elif decl.init == "mixing":
             x = torch.eye(decl.shape[0], decl.shape[1], dtype=torch.float32, device=device) + self.norm_jitter * x
         else:

@@ -349,6 +349,9 @@ class TorchOps:
         x = residual if delta is None else residual + delta_scale * planes_sum(delta)
         return torch.cat([x, origin], dim=1).to(out_dtype)
 
+    def linear_planes_with_spare(self, x, w):
+        return None  # no planes here: the sum is taken by ``accumulate``
+
     def accumulate(self, acc, y):
         acc += planes_sum(y)
         return acc
