@@ -18,8 +18,9 @@ __global__ __launch_bounds__(256) void bias_rotate_pairs_kernel(T* __restrict__ 
   T* row = x + (size_t)t * stride;
   const float pos = freq ? (float)positions[t] : 0.f;
   const int rot_end = freq ? rot_heads * head_dim : 0;
-  // a thread owns columns 2j and 2j + 1; head sizes are even, so a pair never spans two heads
-  for (int j = threadIdx.x; 2 * j < width; j += 256) {
+  // a thread owns columns 2j and 2j + 1; head sizes are even, so a pair never spans two heads.
+  // With few tokens the columns are spread over blocks too (blockIdx.y), one pair a thread.
+  for (int j = blockIdx.y * 256 + threadIdx.x; 2 * j < width; j += 256 * gridDim.y) {
     const int c = 2 * j;
     const bool two = c + 1 < width;
     float u = to_f32<T>(row[c]), v = two ? to_f32<T>(row[c + 1]) : 0.f;
@@ -52,10 +53,12 @@ extern "C" int qrt_bias_rotate_pairs(void* x, long stride, int width, int dtype,
               "bias_rotate_pairs: %d pairs in heads of %d, %d heads in %d columns", pairs, head_dim, rot_heads, width);
   }
   if (num_tokens == 0 || (!bias && !freq)) return 0;
+  const int chunks = num_tokens >= 512 ? 1 : min((width + 511) / 512, 64);
+  const dim3 grid(num_tokens, chunks);
   if (dtype == QRT_F32)
-    bias_rotate_pairs_kernel<float><<<dim3(num_tokens), 256, 0, stream>>>((float*)x, stride, width, bias, positions, freq, rot_heads, head_dim, pairs);
+    bias_rotate_pairs_kernel<float><<<grid, 256, 0, stream>>>((float*)x, stride, width, bias, positions, freq, rot_heads, head_dim, pairs);
   else if (dtype == QRT_BF16)
-    bias_rotate_pairs_kernel<bf16_t><<<dim3(num_tokens), 256, 0, stream>>>((bf16_t*)x, stride, width, bias, positions, freq, rot_heads, head_dim, pairs);
+    bias_rotate_pairs_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)x, stride, width, bias, positions, freq, rot_heads, head_dim, pairs);
   else return qrt_fail("bias_rotate_pairs: unknown dtype %d", dtype);
   QRT_LAUNCH_CHECK("bias_rotate_pairs");
   return 0;

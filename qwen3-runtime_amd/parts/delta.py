@@ -117,6 +117,16 @@ class GatedDeltaRule(Mixer):
             raise ValueError(f"{self._name('q')}: the low-rank pairs' two factors do not fit each other "
                              f"({self.proj.shape[0]} rows in all, {at} expected)")
         self.conv = fetch.constant(torch.cat([fetch.vector_f32(self._name(n) + ".conv") for n, _ in rows[:3]], dim=0))
+        self.second = None
+        if self.a2 is not None and self.g2 is not None:
+            # both low-rank pairs: their second factors as one block-diagonal matrix, so that one
+            # product (float32 out) of the neighbouring columns a1 | g1 serves decay and gate. The
+            # zeros add nothing to either sum.
+            ra, rg = self.decay_rank, self.gate_rank
+            both = torch.zeros((self.a2.shape[0] + self.g2.shape[0], ra + rg), dtype=self.a2.dtype, device=self.a2.device)
+            both[: self.a2.shape[0], :ra] = self.a2
+            both[self.a2.shape[0]:, ra:] = self.g2
+            self.second = fetch.constant(both)
         self.a_log = fetch.vector_f32(self._name("A_log"))
         self.dt_bias = fetch.vector_f32(self._name("dt_bias"))
         self.norm = fetch.vector_f32(self._name("norm"))
@@ -137,17 +147,19 @@ class GatedDeltaRule(Mixer):
         qkv = ops.delta_conv(ctx, y, self.channels, self.conv, tail.state,
                              ((self.kv_heads, self.dim, 2), (self.kv_heads, self.dim, 1), (self.heads, self.vdim, 0)),
                              UNIT_EPS)
-        beta = y[:, cols["b"][0]: cols["b"][0] + self.heads]
-        if self.decay == "head":
-            a = y[:, cols["a"][0]: cols["a"][0] + self.heads]
-        else:  # the decay's logits stay float32 from the second factor on
-            a1 = y[:, cols["a1"][0]: cols["a1"][0] + cols["a1"][1]].contiguous()
-            a = ops.linear(a1, self.a2, out_f32=True)
-        if self.gate == "silu":
-            gate = y[:, cols["g"][0]: cols["g"][0] + self.heads * self.vdim]
+        beta = y[:, cols["b"][0]: cols["b"][0] + self.heads]  # columns of the product, where they lie
+        def columns(name):
+            first, width = cols[name]
+            return y[:, first: first + width]
+
+        if self.second is not None:  # decay logits and gate from one product, float32 out
+            low = y[:, cols["a1"][0]: cols["g1"][0] + cols["g1"][1]].contiguous()
+            both = ops.linear(low, self.second, out_f32=True)
+            a, gate = both[:, : self.heads * self.dim], both[:, self.heads * self.dim:]
         else:
-            g1 = y[:, cols["g1"][0]: cols["g1"][0] + cols["g1"][1]].contiguous()
-            gate = ops.linear(g1, self.g2)
+            # the decay's logits stay float32 from the second factor on
+            a = columns("a") if self.decay == "head" else ops.linear(columns("a1").contiguous(), self.a2, out_f32=True)
+            gate = columns("g") if self.gate == "silu" else ops.linear(columns("g1").contiguous(), self.g2)
         o = ops.delta_rule(ctx, qkv, beta, a, self.a_log, self.dt_bias, state.state, self.heads, self.kv_heads,
                            self.dim, self.vdim, self.decay == "channel")
         out = ops.delta_out(o, self.norm, gate, self.norm_eps, "silu" if self.gate == "silu" else "sigmoid", ctx.dtype)

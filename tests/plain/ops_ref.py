@@ -320,7 +320,7 @@ def delta_rule(qkv, beta, a_logits, a_log, dt_bias, state, cu_q, slots, heads, k
 
 def delta_out(o, weight, gate, eps, gate_kind, out_dtype):
     t, heads, vdim = o.shape
-    z = gate.to(torch.float32).view(t, heads, vdim)
+    z = gate.to(torch.float32).reshape(t, heads, vdim)
     act = z * torch.sigmoid(z) if gate_kind == "silu" else torch.sigmoid(z)
     y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * weight * act
     return y.reshape(t, heads * vdim).to(out_dtype)
