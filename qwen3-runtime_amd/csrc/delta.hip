@@ -483,7 +483,7 @@ extern "C" void qrt_delta_rule_lanes(int lanes) { g_rule_lanes = lanes; }
 extern "C" int qrt_delta_rule(const RuleArgs* args, int num_tokens, int num_seqs, int max_span, hipStream_t stream) {
   RuleArgs a = *args;
   QRT_CHECK(a.heads > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0, "delta_rule: %d heads on %d key heads", a.heads, a.kv_heads);
-  QRT_CHECK(a.dim >= 1 && a.dim <= 256 && a.vdim >= 1, "delta_rule: key size %d (1 to 256), value size %d", a.dim, a.vdim);
+  QRT_CHECK(a.dim >= 1 && a.dim <= 512 && a.vdim >= 1, "delta_rule: key size %d (1 to 512), value size %d", a.dim, a.vdim);
   QRT_CHECK(num_tokens >= 0 && num_seqs >= 0 && num_seqs <= 65535 && a.heads <= 65535, "delta_rule: bad counts");
   QRT_CHECK((uintptr_t)a.state % 16 == 0, "delta_rule: the state is not aligned to 16 bytes");
   if (num_tokens == 0 || num_seqs == 0) return 0;
@@ -499,7 +499,7 @@ extern "C" int qrt_delta_rule(const RuleArgs* args, int num_tokens, int num_seqs
   // Spans of a few tokens (decoding) take tiles of four: a fifth of the LDS, so that four times as
   // many blocks fit a compute unit, and what such a launch waits for is the states' trip from memory.
   const bool few = max_span > 0 && max_span <= 4;
-  const int tokens = few ? 4 : DP <= 128 ? 16 : 8;
+  const int tokens = (few || DP > 256) ? 4 : DP <= 128 ? 16 : 8;
   dim3 grid((a.vdim + cols - 1) / cols, a.heads, num_seqs), block(256);
   const size_t tile = (size_t)tokens * DP * (a.per_channel ? 3 : 2) + (a.per_channel ? 0 : tokens) + 2 * tokens * cols + 2 * tokens;
   const size_t smem = sizeof(float) * 2 * tile;
@@ -509,7 +509,15 @@ extern "C" int qrt_delta_rule(const RuleArgs* args, int num_tokens, int num_seqs
     if (a.per_channel) delta_rule_kernel<GG, true, TT, LL><<<grid, block, smem, stream>>>(a);   \
     else delta_rule_kernel<GG, false, TT, LL><<<grid, block, smem, stream>>>(a);                \
   } while (0)
-  if (few && L == 16) {
+  QRT_CHECK(G <= 8, "delta_rule: %d groups of rows a lane", G);
+  if (L == 16 && G > 4) {  // heads of more than 256 rows: four-token tiles whatever the step
+    switch (G) {
+      case 5: GO(5, 4, 16); break;
+      case 6: GO(6, 4, 16); break;
+      case 7: GO(7, 4, 16); break;
+      default: GO(8, 4, 16); break;
+    }
+  } else if (few && L == 16) {
     switch (G) {
       case 1: GO(1, 4, 16); break;
       case 2: GO(2, 4, 16); break;

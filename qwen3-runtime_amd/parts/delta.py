@@ -47,8 +47,8 @@ class GatedDeltaRule(Mixer):
             raise ValueError(f"unknown decay {decay!r} (head, channel) or gate {gate!r} (silu, sigmoid_low_rank)")
         if not 1 <= int(taps) <= 16:
             raise ValueError(f"the convolution has 1 to 16 taps, not {taps}")
-        if not 1 <= int(head_dim) <= 256:
-            raise ValueError(f"the state's rows are held in registers: key size 1 to 256, not {head_dim}")
+        if not 1 <= int(head_dim) <= 512:
+            raise ValueError(f"the state's rows are held in registers: key size 1 to 512, not {head_dim}")
         self.hidden_size = int(hidden_size)
         self.heads, self.kv_heads = int(num_heads), int(num_kv_heads)
         self.dim, self.vdim = int(head_dim), int(value_dim)

@@ -136,7 +136,7 @@ def plain_rule(q, k, v, beta, a, a_log, dt_bias, per_channel):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("heads,kv_heads,d,dv", [(4, 2, 32, 64), (4, 4, 64, 32), (3, 1, 40, 20), (2, 2, 128, 128), (1, 1, 16, 8),
-                                                 (2, 1, 72, 17), (2, 2, 256, 16), (5, 5, 1, 1)])
+                                                 (2, 1, 72, 17), (2, 2, 256, 16), (5, 5, 1, 1), (1, 1, 320, 24), (2, 1, 512, 8)])
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("sizes", [(300,), (37, 2, 1, 1, 16, 5)])
 def test_delta_rule_against_the_recurrence_written_out(backend, heads, kv_heads, d, dv, per_channel, sizes):
@@ -677,6 +677,58 @@ def test_greedy_generation_through_the_entry_point(folder, name, dtype, graphs):
         below = logits.max(-1).values - logits[range(40), list(tokens)]
         bound = 1e-3 if dtype == "float32" else 2 * NOISE[name] * float(logits.std())
         assert int((below >= bound).sum()) == 0, (float(below.max()), int(below.argmax()))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_command_line_and_trace_replay(folder, tmp_path, dtype):
+    """As a user runs them: ``python -m qwen3_runtime_amd.cli --model DIR`` generates greedily, and
+    ``bin/trace_run`` replays a mixed schedule of seven requests from standard input, four live at
+    most, with a pool that only holds what is live and state slots for four."""
+    import ast
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parents[1]
+    raw, page = config_c()
+    where = folder("c", dtype)
+    cfg, w = P.load(where)
+    prompt = [5, 17, 3, 140, 9, 77, 2]
+    proc = subprocess.run([sys.executable, "-m", "qwen3_runtime_amd.cli", "--model", str(where), "--dtype", dtype,
+                           "--prompt-tokens", *map(str, prompt), "--max-tokens", "8"],
+                          capture_output=True, text=True, timeout=600, cwd=str(root))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = dict(line.split(" ", 1) for line in proc.stdout.splitlines() if " " in line)
+    tokens = ast.literal_eval(lines["runtime"])
+    assert len(tokens) == 8
+    logits = P.forward(cfg, w, prompt + tokens)[len(prompt) - 1: -1]
+    below = logits.max(-1).values - logits[range(8), tokens]
+    assert float(below.max()) < (1e-3 if dtype == "float32" else 2 * NOISE["c"] * float(logits.std()))
+
+    reqs = traces.make_requests(raw["vocab"], [70, 9, 41, 100, 35, 1, 66], seed=6)
+    steps = traces.mixed(reqs, seed=1)
+    out = tmp_path / "logits"
+    proc = subprocess.run([str(root / "bin" / "trace_run"), "--model", str(where), "--dtype", dtype, "--out", str(out),
+                           "--max-tokens", str(traces.peak_tokens(steps))],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True,
+                          timeout=600, cwd=str(root))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert [line for line in proc.stdout.splitlines() if line.startswith("done ")] == [f"done {s['step']}" for s in steps]
+    got, pos = {}, {r: 0 for r in reqs}
+    for s in steps:
+        wanted = sum(len(e["want"]) for e in s["entries"])
+        rows = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(wanted, raw["vocab"]) if wanted else None
+        i = 0
+        for e in s["entries"]:
+            for k in e["want"]:
+                got[(e["id"], pos[e["id"]] + k)] = torch.from_numpy(rows[i].copy())
+                i += 1
+            pos[e["id"]] += len(e["tokens"])
+    check(got, plain_logits(where, reqs), dtype, NOISE["c"])
 
 
 # ------------------------------------------------------------------ configuration and plan
