@@ -528,14 +528,22 @@ def config_d():
                                                "right": delta(1, 1, 100, 36, 3, (1, 2))}, "mlp": moe(12, 1.0, 2, 1, 2, 1)}]}, 8
 
 
-CONFIGS = {"a": config_a, "b": config_b, "c": config_c, "d": config_d}
+def config_e():
+    """Delta rules only: a model without a single page of cache; a loop that runs once."""
+    return {"architecture": "Zisedra", "vocab": 90, "width": 48, "norm": {"eps": 1e-5},
+            "loop": {"start": 0, "stop": 2, "times": 1},
+            "layers": [{"type": "delta", "mixer": delta(2, 1, 16, 16, 4), "mlp": None},
+                       {"type": "delta", "mixer": delta(3, 3, 8, 24, 2), "mlp": moe(16, 1.0, 4, 1, 2, 1)}]}, 16
+
+
+CONFIGS = {"a": config_a, "b": config_b, "c": config_c, "d": config_d, "e": config_e}
 CONFIGS.update({name + "_every": every_expert(make) for name, make in list(CONFIGS.items())})
 # bfloat16: the bound on the largest error of a position's logits, in units of their deviation. The
 # error has a long tail: over six seeds of "c" its median per position was 0.02 and the largest
 # 0.13 to 0.46, at scattered positions; "a" (eight layer runs of width 96, a gain above one at
 # every entry of its loop) measured 0.37, "b" 0.11. float32 showed no error in any of them.
-NOISE = {"a": 0.6, "b": 0.3, "c": 0.6, "d": 0.6}
-LENGTHS = {"a": [1, 7, 45, 130], "b": [3, 17, 50, 64, 101], "c": [2, 16, 17, 120], "d": [1, 5, 40, 83]}
+NOISE = {"a": 0.6, "b": 0.3, "c": 0.6, "d": 0.6, "e": 0.3}
+LENGTHS = {"a": [1, 7, 45, 130], "b": [3, 17, 50, 64, 101], "c": [2, 16, 17, 120], "d": [1, 5, 40, 83], "e": [1, 9, 40, 70]}
 _folders: dict = {}
 
 
@@ -596,7 +604,7 @@ def check(got, want, dtype, noise=0.2):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d", "e"])
 @pytest.mark.parametrize("cut", ["whole", "tail_one_by_one", "portions", "mixed"])
 def test_cuttings_match_plain(folder, backend, name, cut):
     """Whole prompts; the last tokens one by one (across window edges); portions down to two tokens;
@@ -608,6 +616,7 @@ def test_cuttings_match_plain(folder, backend, name, cut):
     loaded = load(folder(name, backend[1]), page, traces.peak_tokens(steps, unit=page) // page, backend)
     got = traces.replay(loaded, steps, poison_freed=True)
     check(got, plain_logits(folder(name, backend[1]), reqs), backend[1], NOISE[name])
+    assert (len(loaded.cache.groups) == 0) == (name == "e")
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
@@ -658,7 +667,7 @@ def test_a_restarted_request_computes_the_same_again(folder, backend):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,graphs", [("float32", False), ("bfloat16", True), ("bfloat16", False)])
-@pytest.mark.parametrize("name", ["a", "c"])
+@pytest.mark.parametrize("name", ["a", "c", "e"])
 def test_greedy_generation_through_the_entry_point(folder, name, dtype, graphs):
     """``LLM.generate`` (scheduler with a small token budget, sampler, graphs where they apply): the
     tokens chosen greedily are, by the plain model given the same context, the best ones or within
