@@ -2,8 +2,12 @@
 // (token, chosen expert) pairs taken one by one.
 //
 // Router: logits z[e] = x . W_r[e] + b[e] in float32 (the router's matrix is held in float32
-// in every mode), the `top` largest per token (ties: the lower index), softmax over those.
-// Experts: pair p = (token t, its j-th expert e) computes act[p] = silu(G_e x) * (U_e x) with
+// in every mode), the `top` largest per token (ties: the lower index), softmax over those; or,
+// with sigmoid scores, the `top` largest sigmoid(z), which weigh the experts as they are. Experts
+// may form equal groups of neighbours of which only the `keep` best (by the sum of a group's two
+// largest entries) stay in the choice.
+// Experts: pair p = (token t, its j-th expert e) computes act[p] = silu(G_e x) * (U_e x) (or the
+// clamped activation of common.h) with
 // gate_up [E, 2I, H] (gate rows, then up rows), then out[t] = sum_j w[t, j] * D_e act[p] with
 // down [E, H, I], float32 out. Every output element is one wave's sum over its row in a fixed
 // order: it depends on neither the batch nor the other pairs. This form streams an expert's

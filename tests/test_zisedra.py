@@ -135,7 +135,7 @@ def plain_rule(q, k, v, beta, a, a_log, dt_bias, per_channel):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("heads,kv_heads,d,dv", [(4, 2, 32, 64), (4, 4, 64, 32), (3, 1, 40, 20), (2, 2, 128, 128), (1, 1, 16, 8),
+@pytest.mark.parametrize("heads,kv_heads,d,dv", [(4, 2, 32, 48), (8, 4, 64, 32), (3, 1, 40, 20), (2, 2, 128, 128), (1, 1, 16, 8),
                                                  (2, 1, 72, 17), (2, 2, 256, 16), (5, 5, 1, 1), (1, 1, 320, 24), (2, 1, 512, 8)])
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("sizes", [(300,), (37, 2, 1, 1, 16, 5)])
@@ -212,7 +212,7 @@ def test_read_out_norm_and_gate(backend, heads, dv, kind):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("heads,kv_heads,d,dims,scaling", [(4, 1, 64, 32, (8.0, 1.0, 4.0, 1024.0)), (3, 3, 16, 16, None),
+@pytest.mark.parametrize("heads,kv_heads,d,dims,scaling", [(4, 1, 64, 24, (6.0, 1.0, 4.0, 512.0)), (3, 3, 16, 16, None),
                                                            (2, 1, 48, 12, (4.0, 1.0, 3.0, 64.0)), (2, 2, 32, 0, None),
                                                            (5, 1, 8, 2, (2.0, 0.5, 2.0, 16.0))])
 def test_pair_rotation_biases_and_scaled_frequencies(backend, heads, kv_heads, d, dims, scaling):
@@ -246,7 +246,7 @@ def test_pair_rotation_biases_and_scaled_frequencies(backend, heads, kv_heads, d
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("experts,top,groups,keep,width", [(16, 2, 2, 1, 320), (12, 3, 3, 2, 96), (6, 2, 1, 1, 64), (8, 4, 8, 4, 50),
+@pytest.mark.parametrize("experts,top,groups,keep,width", [(18, 2, 3, 1, 200), (12, 3, 3, 2, 96), (6, 2, 1, 1, 64), (8, 4, 8, 4, 50),
                                                            (64, 6, 8, 3, 128), (4, 4, 2, 2, 31)])
 def test_router_sigmoid_scores_and_groups(backend, experts, top, groups, keep, width):
     device, dtype = backend
@@ -270,7 +270,7 @@ def test_groups_keep_a_strong_expert_out():
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("experts,top,width,inner,tokens,limit", [(6, 2, 64, 48, 9, 0.8), (16, 2, 320, 64, 3, 1.0), (4, 4, 96, 40, 70, 1.5),
+@pytest.mark.parametrize("experts,top,width,inner,tokens,limit", [(6, 2, 64, 48, 9, 0.8), (16, 2, 256, 96, 3, 1.0), (4, 4, 96, 40, 70, 1.5),
                                                                   (5, 1, 128, 16, 300, 0.5)])
 def test_clamped_experts_weighted_by_their_scores(backend, experts, top, width, inner, tokens, limit):
     """Inputs large enough that the clamps hold on both sides; few pairs, several pairs an expert,
@@ -315,7 +315,7 @@ class DictFetch:
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("width,inner,shared,experts,top,groups,keep", [(128, 64, 128, 8, 2, 2, 1), (320, 64, 128, 16, 2, 2, 1),
+@pytest.mark.parametrize("width,inner,shared,experts,top,groups,keep", [(128, 64, 128, 8, 2, 2, 1), (384, 64, 128, 16, 2, 4, 2),
                                                                         (96, 48, 80, 12, 12, 3, 3), (256, 128, 256, 4, 1, 1, 1)])
 def test_mixture_with_shared_expert_at_every_step_size(backend, width, inner, shared, experts, top, groups, keep):
     """The feed-forward part, routed and shared experts summed, over steps of 1 to 300 tokens: every
@@ -352,7 +352,7 @@ def test_mixture_with_shared_expert_at_every_step_size(backend, width, inner, sh
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("width,tokens,planes", [(96, 5, 1), (320, 3, 4), (2560, 2, 1), (50, 7, 2)])
+@pytest.mark.parametrize("width,tokens,planes", [(96, 5, 1), (352, 3, 4), (2560, 2, 1), (50, 7, 2)])
 def test_scaled_sum_mean_of_norms_and_the_entry_of_a_pass(backend, width, tokens, planes):
     device, dtype = backend
     ops, dt = make_ops(device), DT[dtype]
@@ -379,7 +379,7 @@ def test_scaled_sum_mean_of_norms_and_the_entry_of_a_pass(backend, width, tokens
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("heads,kv_heads,d,dv,window,page,dims", [(4, 1, 64, 64, 72, 16, 32), (2, 2, 32, 16, 9, 8, 32), (6, 2, 16, 16, 21, 16, 4),
+@pytest.mark.parametrize("heads,kv_heads,d,dv,window,page,dims", [(4, 2, 64, 64, 70, 16, 48), (2, 2, 32, 16, 9, 8, 32), (6, 2, 16, 16, 21, 16, 4),
                                                                   (2, 1, 128, 128, 130, 16, 64), (3, 3, 48, 48, 1, 8, 0)])
 def test_window_attention_mixer_sees_a_key_inside_the_window_only(backend, heads, kv_heads, d, dv, window, page, dims):
     """The attention mixer itself (biased projections, pair rotation, window) over a paged cache whose
@@ -490,10 +490,10 @@ def config_b():
 
 def config_c():
     """The whole model is one looped span; head size 64 (decoding through the one-kernel attention)."""
-    return {"architecture": "Zisedra", "vocab": 150, "width": 128, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+    return {"architecture": "Zisedra", "vocab": 150, "width": 128, "norm": {"eps": 1e-5}, "residual_mult": 0.6,
             "loop": {"start": 0, "stop": 2, "times": 2},
             "layers": [
-                {"type": "parallel", "mixer": {"left": window(2, 1, 64, 64, 0.125, 50, 32, 250000.0, (8.0, 1.0, 4.0, 1024.0)),
+                {"type": "parallel", "mixer": {"left": window(2, 1, 64, 64, 0.11, 50, 48, 100000.0, (8.0, 1.0, 4.0, 2048.0)),
                                                "right": delta(2, 1, 128, 64, 4, (16, 16))}, "mlp": moe(64, 1.0, 4, 2, 2, 1, (64, 1.0))},
                 {"type": "delta", "mixer": delta(1, 1, 64, 128, 2), "mlp": None}]}, 16
 
