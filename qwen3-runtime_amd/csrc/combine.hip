@@ -11,11 +11,32 @@ struct Planes {
   const void* p; int code; int planes; long plane_stride;
 };
 
+// Up to eight planes are asked for together (a plane that is not there: the first one again, dropped),
+// so that an element costs one trip to memory however many planes it has; they are added in order.
 __device__ __forceinline__ float planes_at(const Planes& y, size_t i) {
   if (y.code == QRT_BF16) return (float)((const bf16_t*)y.p)[i];
+  const float* p = (const float*)y.p;
+  if (y.planes == 1) return p[i];
+  float part[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) part[k] = p[(size_t)(k < y.planes ? k : 0) * y.plane_stride + i];
   float v = 0.f;
-  for (int k = 0; k < y.planes; ++k) v += ((const float*)y.p)[(size_t)k * y.plane_stride + i];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v += k < y.planes ? part[k] : 0.f;
+  for (int k = 8; k < y.planes; ++k) v += p[(size_t)k * y.plane_stride + i];
   return v;
+}
+
+// Two sums over a block of up to 1,024 threads at once; every thread gets both.
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  if (lane == 0) { red[wave] = a; red[16 + wave] = b; }
+  __syncthreads();
+  a = b = 0.f;
+  for (int i = 0; i < nw; ++i) { a += red[i]; b += red[16 + i]; }  // the same order in every thread
 }
 
 // out[t] = (1/2) (a[t] / rms(a[t]) * wa + b[t] / rms(b[t]) * wb), rms with eps inside the root.
@@ -49,8 +70,9 @@ __global__ __launch_bounds__(1024) void norm_mean_kernel(Planes ya, Planes yb, c
     sa += x * x;
     sb += y * y;
   }
-  const float ia = 1.0f / sqrtf(block_sum(sa, red) / (float)hidden + eps);
-  const float ib = 1.0f / sqrtf(block_sum(sb, red) / (float)hidden + eps);
+  block_sum2(sa, sb, red);
+  const float ia = 1.0f / sqrtf(sa / (float)hidden + eps);
+  const float ib = 1.0f / sqrtf(sb / (float)hidden + eps);
 #pragma unroll
   for (int j = 0; j < NM_KEEP; ++j) {
     const int i = threadIdx.x + 1024 * j;
