@@ -536,14 +536,34 @@ def config_e():
                        {"type": "delta", "mixer": delta(3, 3, 8, 24, 2), "mlp": moe(16, 1.0, 4, 1, 2, 1)}]}, 16
 
 
-CONFIGS = {"a": config_a, "b": config_b, "c": config_c, "d": config_d, "e": config_e}
+def config_f():
+    """Sizes that are multiples of nothing: width 90, values of 7 and 5 elements, keys of 10, 6 and 3,
+    experts of 9 and 5, a shared expert of 11."""
+    return {"architecture": "Zisedra", "vocab": 77, "width": 90, "norm": {"eps": 1e-5}, "residual_mult": 0.9,
+            "loop": {"start": 0, "stop": 1, "times": 2},
+            "layers": [{"type": "parallel", "mixer": {"left": window(3, 1, 10, 7, 0.3, 13, 6, 50.0), "right": delta(2, 1, 6, 5, 3, (3, 2))},
+                        "mlp": moe(9, 1.0, 3, 2, 1, 1, (11, 1.0))},
+                       {"type": "delta", "mixer": delta(5, 5, 3, 9, 2), "mlp": moe(5, 0.5, 2, 1, 2, 1)}]}, 8
+
+
+def config_g():
+    """Layers of a real model's proportions (heads of 128, a window of 256, experts of 512): the kernel
+    forms that small sizes never reach."""
+    return {"architecture": "Zisedra", "vocab": 500, "width": 1024, "norm": {"eps": 1e-5}, "residual_mult": 0.8,
+            "layers": [{"type": "delta", "mixer": delta(8, 2, 128, 128, 4), "mlp": moe(512, 2.0, 8, 2, 4, 2, (512, 2.0))},
+                       {"type": "parallel", "mixer": {"left": window(8, 2, 128, 128, 0.09, 256, 64, 10000.0),
+                                                      "right": delta(8, 2, 128, 128, 4, (32, 32))},
+                        "mlp": moe(512, 2.0, 8, 2, 4, 2, (512, 2.0))}]}, 16
+
+
+CONFIGS = {"a": config_a, "b": config_b, "c": config_c, "d": config_d, "e": config_e, "f": config_f, "g": config_g}
 CONFIGS.update({name + "_every": every_expert(make) for name, make in list(CONFIGS.items())})
 # bfloat16: the bound on the largest error of a position's logits, in units of their deviation. The
 # error has a long tail: over six seeds of "c" its median per position was 0.02 and the largest
 # 0.13 to 0.46, at scattered positions; "a" (eight layer runs of width 96, a gain above one at
 # every entry of its loop) measured 0.37, "b" 0.11. float32 showed no error in any of them.
-NOISE = {"a": 0.6, "b": 0.3, "c": 0.6, "d": 0.6, "e": 0.3}
-LENGTHS = {"a": [1, 7, 45, 130], "b": [3, 17, 50, 64, 101], "c": [2, 16, 17, 120], "d": [1, 5, 40, 83], "e": [1, 9, 40, 70]}
+NOISE = {"a": 0.6, "b": 0.3, "c": 0.6, "d": 0.6, "e": 0.3, "f": 0.6, "g": 0.3}
+LENGTHS = {"a": [1, 7, 45, 130], "b": [3, 17, 50, 64, 101], "c": [2, 16, 17, 120], "d": [1, 5, 40, 83], "e": [1, 9, 40, 70], "f": [1, 9, 40, 70]}
 _folders: dict = {}
 
 
@@ -557,7 +577,7 @@ def folder(tmp_path_factory):
         if name not in _folders:
             raw, _ = CONFIGS[name]()
             _folders[name] = write_model_folder(tmp_path_factory.mktemp("zisedra_" + name), raw, seed=71 + len(_folders),
-                                                std=0.08, norm_jitter=0.2)
+                                                std=0.03 if name.startswith("g") else 0.08, norm_jitter=0.2)
         return _folders[name]
 
     return get
@@ -604,7 +624,7 @@ def check(got, want, dtype, noise=0.2):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["a", "b", "c", "d", "e"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d", "e", "f"])
 @pytest.mark.parametrize("cut", ["whole", "tail_one_by_one", "portions", "mixed"])
 def test_cuttings_match_plain(folder, backend, name, cut):
     """Whole prompts; the last tokens one by one (across window edges); portions down to two tokens;
@@ -617,6 +637,19 @@ def test_cuttings_match_plain(folder, backend, name, cut):
     got = traces.replay(loaded, steps, poison_freed=True)
     check(got, plain_logits(folder(name, backend[1]), reqs), backend[1], NOISE[name])
     assert (len(loaded.cache.groups) == 0) == (name == "e")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_a_real_model_s_proportions(folder, dtype):
+    """A 330-token prompt in one step, then in portions with its last tokens one by one, beside a
+    second request: prompt kernels with full tiles, the window passing, experts by expert."""
+    raw, page = config_g()
+    reqs = traces.make_requests(raw["vocab"], [330, 40], seed=9)
+    want = plain_logits(folder("g", dtype), reqs)
+    for steps in (traces.whole(reqs), traces.mixed(reqs, seed=2, decode_tail=12)):
+        loaded = load(folder("g", dtype), page, traces.peak_tokens(steps, unit=page) // page, ("cuda:0", dtype))
+        check(traces.replay(loaded, steps, poison_freed=True), want, dtype, NOISE["g"])
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
