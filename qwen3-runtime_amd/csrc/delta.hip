@@ -234,12 +234,12 @@ extern "C" int qrt_delta_conv(const ConvArgs* args, int dtype, int num_seqs, int
 }
 
 // ------------------------------------------------------------------ the recurrence
-// A block of 256 threads owns 16 value channels (columns of S) of one head of one sequence and
-// walks the span's tokens in order. A column is shared by 16 neighbouring lanes: lane l holds
-// the rows 4l .. 4l+3, 64 + 4l .. 64 + 4l+3, ... (R of them, four neighbours at a time: one
+// A block of 256 threads owns 16 (or 32) value channels (columns of S) of one head of one sequence
+// and walks the span's tokens in order. A column is shared by L = 16 (or 8) neighbouring lanes:
+// lane l holds the rows 4l .. 4l+3, 4L + 4l .. 4L + 4l+3, ... (four neighbours at a time: one
 // 16-byte access to memory or LDS) in registers, so the two sums over rows that a token
-// needs, S^T k and S^T q, are sums inside a row of 16 lanes (four DPP steps each, no LDS), and
-// they run side by side: the read-out is taken from the decayed state, before the write, and
+// needs, S^T k and S^T q, are sums inside a row of lanes (four or three DPP steps each, no LDS),
+// and they run side by side: the read-out is taken from the decayed state, before the write, and
 // completed by (k . q) u, which is the write's share of it.
 // Tokens are staged through LDS 16 at a time, in two buffers: while the block walks one tile its
 // threads hold the next tile's keys, queries, decay logits, values and step-size logits in
@@ -496,7 +496,7 @@ extern "C" int qrt_delta_rule(const RuleArgs* args, int num_tokens, int num_seqs
   if (L != 8 && L != 16) L = ((long)num_seqs * a.heads * ((a.vdim + 31) / 32) >= 1024 && a.dim <= 128) ? 8 : 16;
   if (a.dim > 128) L = 16;
   const int G = (a.dim + 4 * L - 1) / (4 * L), DP = 4 * L * G, cols = 256 / L;
-  // Spans of a few tokens (decoding) take tiles of four: a fifth of the LDS, so that four times as
+  // Spans of a few tokens (decoding) take tiles of four: a quarter of the LDS, so that four times as
   // many blocks fit a compute unit, and what such a launch waits for is the states' trip from memory.
   const bool few = max_span > 0 && max_span <= 4;
   const int tokens = (few || DP > 256) ? 4 : DP <= 128 ? 16 : 8;
